@@ -613,20 +613,31 @@ int vlm_linear_recurrence(const vlm_recurrence_args* a, int nseg, int ntok, int 
 
 /* csrc/latent_attn.hip: pool T [pages][64][R + Dr]; token t belongs to block-table row tok_seq[t] at position tok_pos[t] */
 int vlm_latent_kv_write(const void* d, long ldd, const void* w, int R, int Dr, const void* inv_freq, const void* tok_seq,
-                        const void* tok_pos, const void* block_table, int max_pages, void* pool, float eps, int rows, int dtype,
-                        void* stream);
+                        const void* tok_pos, const void* block_table, int max_pages, void* pool, float eps, int rot_half, int rows,
+                        int dtype, void* stream);
+/* rot_half (both functions above and below): 0 = the rotated pairs are (2 i, 2 i + 1), 1 = (i, i + Dr / 2).  ABI v11. */
 int vlm_rope_pairs_rows(const void* q, long ldq, long head_stride, int H, int Dr, const void* inv_freq, const void* tok_pos, void* out,
-                        long ldo, long out_head_stride, int rows, int dtype, void* stream);
+                        long ldo, long out_head_stride, int rot_half, int rows, int dtype, void* stream);
+/* window > 0 (ABI v11): query i sees the keys j with 0 <= i - j < window; <= 0: every j <= i */
 int vlm_latent_attn(const void* q, const void* pool, const void* tok_seq, const void* tok_pos, const void* block_table, int max_pages,
-                    int H, int R, int Dr, float scale, const void* gate, long ldgate, void* out, int rows, int dtype, void* stream);
+                    int H, int R, int Dr, float scale, int window, const void* gate, long ldgate, void* out, int rows, int dtype,
+                    void* stream);
 /* the prompt form: query blocks (first token, count <= 16, all of one sequence and consecutive) x heads, key tiles through LDS;
  * R <= 512.  Same results as vlm_latent_attn up to summation order. */
 int vlm_latent_attn_blocks(const void* q, const void* pool, const void* qb_start, const void* qb_count, int nblocks, const void* tok_seq,
-                           const void* tok_pos, const void* block_table, int max_pages, int H, int R, int Dr, float scale,
+                           const void* tok_pos, const void* block_table, int max_pages, int H, int R, int Dr, float scale, int window,
                            const void* gate, long ldgate, void* out, int dtype, void* stream);
 
 /* csrc/moe.hip */
 int vlm_moe_route(const void* logits, int T, int E, int top, void* gate, void* idx, void* wgt, void* stream);
+/* ABI v11.  The same choice and outputs with weights = softmax over ALL experts * scale (not renormalised), limited to the experts
+ * of the `keep` best of `groups` equal groups of neighbours (a group's score: its largest member; groups <= 64). */
+int vlm_moe_route_scored(const void* logits, int T, int E, int top, int groups, int keep, float scale, void* gate, void* idx, void* wgt,
+                         void* stream);
+/* ABI v11.  out[t][c] = act(g[t][c]) * u[t][c], act 0 = tanh-form gelu, 1 = silu, 2 = sigmoid; with route (fp32 [rows][E]): E stacked
+ * experts of ff columns, the columns of expert e in g / u start at e * estride, times route[t][e] (a zero writes an exact zero). */
+int vlm_glu_rows(const void* g, long ldg, const void* u, long ldu, const void* route, int E, int ff, int estride, int act, void* out,
+                 long ldo, int rows, int dim, int dtype, void* stream);
 int vlm_moe_relu2_gate(const void* up, long ldu, const void* gate, int E, int ff, int shared, void* out, long ldo, int rows, int dtype,
                        void* stream);
 
@@ -638,6 +649,10 @@ int vlm_rms_rows(const void* x, const void* w, void* out, int rows, int D, long 
 int vlm_gated_rms_add(void* x, const void* a, long lda, const void* wa, const void* b, long ldb, const void* wb, const void* gate,
                       long ldg, const void* gate_bias, const void* w, void* h, int rows, int D, float eps, int dtype, void* stream);
 int vlm_relu2_rows(const void* in, long ldi, void* out, long ldo, int rows, int dim, int dtype, void* stream);
+/* ABI v11.  x[t] += mult * y[t] (y T rows at ldy, may be NULL), then h[t] = rms(x[t]) * (w_offset + w) into T rows at ldh (w may be
+ * NULL: no norm).  The residual step of a pre-norm sublayer fused with the norm of the next reader. */
+int vlm_scaled_add_rms(void* x, const void* y, long ldy, float mult, const void* w, float w_offset, void* h, long ldh, int rows, int D,
+                       float eps, int dtype, void* stream);
 
 /* csrc/delta_rule.hip: delta-rule recurrences (the update reads the old state), state fp32 [slots][H][D][Dv].
  * Prepare passes write fp32 rows; the scan + finish take them.  Segments as in vlm_linear_recurrence. */
@@ -691,17 +706,41 @@ typedef struct vlm_delta_rule_args {
 int vlm_delta_rule(const vlm_delta_rule_args* a, int nseg, int ntok, int dtype, void* stream);
 
 /* csrc/window_attn.hip: grouped-head softmax attention with a sliding window over paged caches: keys fp32 [pages][64][KH * D]
- * (normed, rotated), values T [pages][64][KH * Dv].  window <= 0: causal without a window.  temp: T [H] or NULL. */
+ * (normed, rotated), values T [pages][64][KH * Dv].  window <= 0: causal without a window.  temp: T [H] or NULL.
+ * ABI v11: cap > 0: scores pass cap * tanh(. / cap); gate_head: the gate is one number per head (T [.][H] at ldgate) instead of
+ * one per value column. */
+typedef struct vlm_headnorm_args {
+  const void* x;                        /* T rows [heads * D] at ldx */
+  long ldx;
+  int heads, D;
+  const void* bias;                     /* T [heads * D] or NULL, added first */
+  const void* w;                        /* T [D] or NULL */
+  int norm;                             /* 0 = none, 1 = per-head RMS norm (times w when given) */
+  float eps;
+  int rot_dims;                         /* pairs (2 i, 2 i + 1) of the first rot_dims dimensions */
+  const float* inv_freq;
+  float temp_coef;                      /* temp_every > 0: times 1 + temp_coef * ln(floor((pos + 1) / temp_every) + 1) */
+  int temp_every;
+  const int *tok_pos, *tok_seq, *block_table;   /* block_table NULL: dense output rows */
+  int max_pages;
+  float* out;
+  const void* raw;                      /* T rows [heads * Draw] at ldraw (+ raw_bias T [heads * Draw]) copied into raw_pool (T) */
+  long ldraw;
+  int Draw;
+  const void* raw_bias;
+  void* raw_pool;
+} vlm_headnorm_args;
+int vlm_headnorm_rows(const vlm_headnorm_args* a, int rows, int dtype, void* stream);
 int vlm_headnorm_rope_rows(const void* x, long ldx, int heads, int D, const void* w, float eps, int rot_dims, const void* inv_freq,
                            const void* tok_pos, const void* tok_seq, const void* block_table, int max_pages, void* out, void* raw_pool,
                            int rows, int dtype, void* stream);
 int vlm_window_attn_blocks(const void* q, const void* kpool, const void* vpool, const void* qb_start, const void* qb_count, int nblocks,
                            const void* tok_seq, const void* tok_pos, const void* block_table, int max_pages, int H, int KH, int D, int Dv,
-                           float scale, const void* temp, int window, const void* gate, long ldgate, void* out, long ldo, int dtype,
-                           void* stream);
+                           float scale, const void* temp, int window, float cap, const void* gate, long ldgate, int gate_head, void* out,
+                           long ldo, int dtype, void* stream);
 int vlm_window_attn_rows(const void* q, const void* kpool, const void* vpool, const void* tok_seq, const void* tok_pos,
                          const void* block_table, int max_pages, int H, int KH, int D, int Dv, float scale, const void* temp, int window,
-                         const void* gate, long ldgate, void* out, long ldo, int rows, int dtype, void* stream);
+                         float cap, const void* gate, long ldgate, int gate_head, void* out, long ldo, int rows, int dtype, void* stream);
 
 #ifdef __cplusplus
 }

@@ -126,6 +126,14 @@ class DeltaRuleArgs(C.Structure):
                    ("H", c_int), ("KH", c_int), ("D", c_int), ("Dv", c_int)])
 
 
+class HeadnormArgs(C.Structure):
+    """vlm_headnorm_args (include/vlm_hip.h)"""
+    _fields_ = [("x", c_void_p), ("ldx", C.c_long), ("heads", c_int), ("D", c_int), ("bias", c_void_p), ("w", c_void_p), ("norm", c_int),
+                ("eps", c_float), ("rot_dims", c_int), ("inv_freq", c_void_p), ("temp_coef", c_float), ("temp_every", c_int),
+                ("tok_pos", c_void_p), ("tok_seq", c_void_p), ("block_table", c_void_p), ("max_pages", c_int), ("out", c_void_p),
+                ("raw", c_void_p), ("ldraw", C.c_long), ("Draw", c_int), ("raw_bias", c_void_p), ("raw_pool", c_void_p)]
+
+
 DECODE_FUSED_TAIL = 1                       # vlm_decode_args.flags
 DECODE_ACT16 = 2                            # `act` holds 16 x intermediate_size elements (tiled hand-over to the down projection)
 TUNE_MFMA_GEMV, TUNE_ATTN_PAGESPLIT, TUNE_GEMV_VARIANT, TUNE_ATTN_MERGE = 6, 7, 8, 9  # vlm_llm_set_tuning keys (include/vlm_hip.h)
@@ -217,13 +225,19 @@ SIGNATURES = {
                                         c_int, c_int, c_void_p]),
     "vlm_linear_recurrence": (c_int, [P(RecurrenceArgs), c_int, c_int, c_int, c_void_p]),
     "vlm_latent_kv_write": (c_int, [c_void_p, C.c_long, c_void_p, c_int, c_int] + [c_void_p] * 4 + [c_int, c_void_p, c_float, c_int,
-                                    c_int, c_void_p]),
-    "vlm_rope_pairs_rows": (c_int, [c_void_p, C.c_long, C.c_long, c_int, c_int, c_void_p, c_void_p, c_void_p, C.c_long, C.c_long,
                                     c_int, c_int, c_void_p]),
-    "vlm_latent_attn": (c_int, [c_void_p] * 5 + [c_int] * 4 + [c_float, c_void_p, C.c_long, c_void_p, c_int, c_int, c_void_p]),
-    "vlm_latent_attn_blocks": (c_int, [c_void_p] * 4 + [c_int] + [c_void_p] * 3 + [c_int] * 4 + [c_float, c_void_p, C.c_long, c_void_p,
-                                       c_int, c_void_p]),
+    "vlm_rope_pairs_rows": (c_int, [c_void_p, C.c_long, C.c_long, c_int, c_int, c_void_p, c_void_p, c_void_p, C.c_long, C.c_long,
+                                    c_int, c_int, c_int, c_void_p]),
+    "vlm_latent_attn": (c_int, [c_void_p] * 5 + [c_int] * 4 + [c_float, c_int, c_void_p, C.c_long, c_void_p, c_int, c_int, c_void_p]),
+    "vlm_latent_attn_blocks": (c_int, [c_void_p] * 4 + [c_int] + [c_void_p] * 3 + [c_int] * 4 + [c_float, c_int, c_void_p, C.c_long,
+                                       c_void_p, c_int, c_void_p]),
     "vlm_moe_route": (c_int, [c_void_p, c_int, c_int, c_int, c_void_p, c_void_p, c_void_p, c_void_p]),
+    "vlm_moe_route_scored": (c_int, [c_void_p, c_int, c_int, c_int, c_int, c_int, c_float, c_void_p, c_void_p, c_void_p, c_void_p]),
+    "vlm_glu_rows": (c_int, [c_void_p, C.c_long, c_void_p, C.c_long, c_void_p, c_int, c_int, c_int, c_int, c_void_p, C.c_long, c_int,
+                             c_int, c_int, c_void_p]),
+    "vlm_scaled_add_rms": (c_int, [c_void_p, c_void_p, C.c_long, c_float, c_void_p, c_float, c_void_p, C.c_long, c_int, c_int, c_float,
+                                   c_int, c_void_p]),
+    "vlm_headnorm_rows": (c_int, [P(HeadnormArgs), c_int, c_int, c_void_p]),
     "vlm_moe_relu2_gate": (c_int, [c_void_p, C.c_long, c_void_p, c_int, c_int, c_int, c_void_p, C.c_long, c_int, c_int, c_void_p]),
     "vlm_stream_cast": (c_int, [c_void_p, c_void_p, c_int, c_int, c_int, c_void_p]),
     "vlm_rms_rows": (c_int, [c_void_p] * 3 + [c_int, c_int, C.c_long, c_float, c_int, c_void_p]),
@@ -235,10 +249,10 @@ SIGNATURES = {
     "vlm_delta_rule": (c_int, [P(DeltaRuleArgs), c_int, c_int, c_int, c_void_p]),
     "vlm_headnorm_rope_rows": (c_int, [c_void_p, C.c_long, c_int, c_int, c_void_p, c_float, c_int] + [c_void_p] * 4 + [c_int, c_void_p,
                                        c_void_p, c_int, c_int, c_void_p]),
-    "vlm_window_attn_blocks": (c_int, [c_void_p] * 5 + [c_int] + [c_void_p] * 3 + [c_int] * 5 + [c_float, c_void_p, c_int, c_void_p,
-                                       C.c_long, c_void_p, C.c_long, c_int, c_void_p]),
-    "vlm_window_attn_rows": (c_int, [c_void_p] * 6 + [c_int] * 5 + [c_float, c_void_p, c_int, c_void_p, C.c_long, c_void_p, C.c_long,
-                                     c_int, c_int, c_void_p]),
+    "vlm_window_attn_blocks": (c_int, [c_void_p] * 5 + [c_int] + [c_void_p] * 3 + [c_int] * 5 + [c_float, c_void_p, c_int, c_float,
+                                       c_void_p, C.c_long, c_int, c_void_p, C.c_long, c_int, c_void_p]),
+    "vlm_window_attn_rows": (c_int, [c_void_p] * 6 + [c_int] * 5 + [c_float, c_void_p, c_int, c_float, c_void_p, C.c_long, c_int,
+                                     c_void_p, C.c_long, c_int, c_int, c_void_p]),
 }
 
 _lib = None

@@ -7,14 +7,17 @@
 // and attention runs straight over the cached rows [c | kr] with "head dim" R + Dr for scores and R for values; nothing
 // per head is ever cached or materialised per key.  A layer may read ANOTHER layer's cache (same R, Dr, rotation).
 //
-//   vlm_latent_kv_write      d = W_dkv h rows -> c = d[:R] * rsqrt(mean(d[:R]^2) + eps) * w, kr = rope_pairs(d[R:], pos) into the
+//   vlm_latent_kv_write      d = W_dkv h rows -> c = d[:R] * rsqrt(mean(d[:R]^2) + eps) * w, kr = rope(d[R:], pos) into the
 //                            paged pool [page][64][R + Dr] (T-typed) of the token's sequence
-//   vlm_rope_pairs_rows      rotate the Dr-wide rotary part of every head's query (pairs (2 i, 2 i + 1)) into the fp32 query
-//                            buffer behind the absorbed part
+//   vlm_rope_pairs_rows      rotate the Dr-wide rotary part of every head's query into the fp32 query buffer behind the
+//                            absorbed part
+//                            (both: pairs (2 i, 2 i + 1), or with rot_half the pairs (i, i + Dr / 2))
 //   vlm_latent_attn          causal softmax attention of fp32 queries [T][H][R + Dr] over the pool; key tiles start at
 //                            multiples of 256 counted from the sequence's first token, so the arithmetic of a token does not
 //                            depend on how its prompt was cut; output fp32 [T][H][R], times sigmoid(gate[t][h]) when a gate
 //                            is given
+// A sliding window (window > 0) limits query i to the keys j with 0 <= i - j < window; tiles still sit at multiples of their
+// size counted from the sequence's first token and start at the tile that holds the window's edge.
 // Scores, softmax and the weighted sum are fp32.  dtype: 0 = bf16, 1 = fp32 for the T-typed pointers.
 #include "common.hpp"
 #include "../../include/vlm_hip.h"
@@ -34,7 +37,7 @@ template <typename T>
 __global__ __launch_bounds__(256) void latent_kv_write_kernel(const T* __restrict__ d, long ldd, const T* __restrict__ w, int R, int Dr,
                                                               const float* __restrict__ inv_freq, const int* __restrict__ tok_seq,
                                                               const int* __restrict__ tok_pos, const int* __restrict__ block_table,
-                                                              int max_pages, T* __restrict__ pool, float eps) {
+                                                              int max_pages, T* __restrict__ pool, float eps, int rot_half) {
   __shared__ float red[4];
   const long t = blockIdx.x;
   const T* row = d + t * ldd;
@@ -53,30 +56,33 @@ __global__ __launch_bounds__(256) void latent_kv_write_kernel(const T* __restric
   const float r = 1.0f / sqrtf(((red[0] + red[1]) + (red[2] + red[3])) / (float)R + eps);
   for (int i = threadIdx.x; i < R; i += 256) st_f(dst + i, ld_f(row + i) * r * ld_f(w + i));
   for (int i = threadIdx.x; i < Dr / 2; i += 256) {
-    const float u = ld_f(row + R + 2 * i), v = ld_f(row + R + 2 * i + 1);
+    const int i0 = rot_half ? i : 2 * i, i1 = rot_half ? i + Dr / 2 : 2 * i + 1;
+    const float u = ld_f(row + R + i0), v = ld_f(row + R + i1);
     float sn, cs;
     sincosf((float)pos * inv_freq[i], &sn, &cs);
-    st_f(dst + R + 2 * i, u * cs - v * sn);
-    st_f(dst + R + 2 * i + 1, v * cs + u * sn);
+    st_f(dst + R + i0, u * cs - v * sn);
+    st_f(dst + R + i1, v * cs + u * sn);
   }
 }
 
 template <typename T>
 __global__ __launch_bounds__(256) void rope_pairs_rows_kernel(const T* __restrict__ q, long ldq, long head_stride, int H, int Dr,
                                                               const float* __restrict__ inv_freq, const int* __restrict__ tok_pos,
-                                                              float* __restrict__ out, long ldo, long out_head_stride, int rows) {
+                                                              float* __restrict__ out, long ldo, long out_head_stride, int rows,
+                                                              int rot_half) {
   const long i = (long)blockIdx.x * 256 + threadIdx.x;
   const int hp = Dr / 2;
   if (i >= (long)rows * H * hp) return;
   const int pi = (int)(i % hp), h = (int)((i / hp) % H);
   const long t = i / ((long)hp * H);
   const T* src = q + t * ldq + (long)h * head_stride;
-  const float u = ld_f(src + 2 * pi), v = ld_f(src + 2 * pi + 1);
+  const int i0 = rot_half ? pi : 2 * pi, i1 = rot_half ? pi + hp : 2 * pi + 1;
+  const float u = ld_f(src + i0), v = ld_f(src + i1);
   float sn, cs;
   sincosf((float)tok_pos[t] * inv_freq[pi], &sn, &cs);
   float* dst = out + t * ldo + (long)h * out_head_stride;
-  dst[2 * pi] = u * cs - v * sn;
-  dst[2 * pi + 1] = v * cs + u * sn;
+  dst[i0] = u * cs - v * sn;
+  dst[i1] = v * cs + u * sn;
 }
 
 // workgroup = (token, head): one key per lane and tile for the scores, one value dimension per lane for the weighted sum
@@ -84,7 +90,7 @@ template <typename T, int NACC>
 __global__ __launch_bounds__(256) void latent_attn_kernel(const float* __restrict__ q, const T* __restrict__ pool,
                                                           const int* __restrict__ tok_seq, const int* __restrict__ tok_pos,
                                                           const int* __restrict__ block_table, int max_pages, int H, int R, int Dr,
-                                                          float scale, const T* __restrict__ gate, long ldgate,
+                                                          float scale, int window, const T* __restrict__ gate, long ldgate,
                                                           float* __restrict__ out) {
   extern __shared__ float smem[];
   const int Dk = R + Dr;
@@ -102,10 +108,11 @@ __global__ __launch_bounds__(256) void latent_attn_kernel(const float* __restric
 #pragma unroll
   for (int a = 0; a < NACC; ++a) acc[a] = 0.f;
   const int nkeys = pos + 1;
-  for (int j0 = 0; j0 < nkeys; j0 += 256) {
+  const int first = window > 0 ? max(0, pos - window + 1) : 0;          // the oldest visible key
+  for (int j0 = (first / 256) * 256; j0 < nkeys; j0 += 256) {
     const int j = j0 + tid;
     float s = -INFINITY;
-    if (j < nkeys) {
+    if (j < nkeys && j >= first) {
       const T* kr = pool + ((long)bt[j / PAGE] * PAGE + j % PAGE) * Dk;
       float d = 0.f;
       for (int i = 0; i < Dk; ++i) d = fmaf(qs[i], ld_f(kr + i), d);
@@ -117,7 +124,7 @@ __global__ __launch_bounds__(256) void latent_attn_kernel(const float* __restric
     if ((tid & 63) == 0) red[tid >> 6] = mx;
     __syncthreads();
     const float m_new = fmaxf(m_run, fmaxf(fmaxf(red[0], red[1]), fmaxf(red[2], red[3])));
-    const float pj = j < nkeys ? expf(s - m_new) : 0.f;
+    const float pj = (j < nkeys && j >= first) ? expf(s - m_new) : 0.f;
     ps[tid] = pj;
     float sum = pj;
 #pragma unroll
@@ -133,7 +140,7 @@ __global__ __launch_bounds__(256) void latent_attn_kernel(const float* __restric
       const int dcol = tid + a * 256;
       if (dcol < R) {
         float v = acc[a] * alpha;
-        for (int jj = 0; jj < nk; ++jj) {
+        for (int jj = max(0, first - j0); jj < nk; ++jj) {
           const int key = j0 + jj;
           v = fmaf(ps[jj], ld_f(pool + ((long)bt[key / PAGE] * PAGE + key % PAGE) * Dk + dcol), v);
         }
@@ -175,8 +182,8 @@ __global__ __launch_bounds__(256) void latent_attn_block_kernel(const float* __r
                                                                 const int* __restrict__ qb_start, const int* __restrict__ qb_count,
                                                                 const int* __restrict__ tok_seq, const int* __restrict__ tok_pos,
                                                                 const int* __restrict__ block_table, int max_pages, int H, int R,
-                                                                int Dr, float scale, const T* __restrict__ gate, long ldgate,
-                                                                float* __restrict__ out) {
+                                                                int Dr, float scale, int window, const T* __restrict__ gate,
+                                                                long ldgate, float* __restrict__ out) {
   extern __shared__ float smem[];
   const int Dk = R + Dr, DP = (Dk + 7) & ~7, KP = DP + 4;
   float* qs = smem;                         // [QB][DP]
@@ -202,7 +209,8 @@ __global__ __launch_bounds__(256) void latent_attn_block_kernel(const float* __r
     for (int b = 0; b < NACC; ++b) acc[a][b] = 0.f;
   const int nkeys = pos0 + nq;              // the last query sees keys 0 .. pos0 + nq - 1
   const bool vec = (Dk & 7) == 0;           // rows of the pool are 16-byte aligned and a whole number of 8-element groups
-  for (int j0 = 0; j0 < nkeys; j0 += KT) {
+  const int first = window > 0 ? max(0, pos0 - window + 1) : 0;        // the first query's oldest visible key
+  for (int j0 = (first / KT) * KT; j0 < nkeys; j0 += KT) {
     __syncthreads();                        // (qs / state initialised; the previous tile's ks and ps are no longer read)
     {
       const int key = j0 + r16;
@@ -236,7 +244,8 @@ __global__ __launch_bounds__(256) void latent_attn_block_kernel(const float* __r
         d = fmaf(a.z, b.z, d);
         d = fmaf(a.w, b.w, d);
       }
-      const bool seen = r16 < nq && j0 + l16 <= pos0 + r16;
+      const int dist = pos0 + r16 - (j0 + l16);
+      const bool seen = r16 < nq && dist >= 0 && (window <= 0 || dist < window);
       ps[l16 * QB + r16] = seen ? d * scale : -INFINITY;
     }
     __syncthreads();
@@ -301,8 +310,8 @@ __global__ __launch_bounds__(256) void latent_attn_block_kernel(const float* __r
 }  // namespace
 
 extern "C" int vlm_latent_kv_write(const void* d, long ldd, const void* w, int R, int Dr, const void* inv_freq, const void* tok_seq,
-                                   const void* tok_pos, const void* block_table, int max_pages, void* pool, float eps, int rows,
-                                   int dtype, void* stream) {
+                                   const void* tok_pos, const void* block_table, int max_pages, void* pool, float eps, int rot_half,
+                                   int rows, int dtype, void* stream) {
   if (!d || !w || !tok_seq || !tok_pos || !block_table || !pool || R <= 0 || Dr < 0 || (Dr & 1) || (Dr && !inv_freq) ||
       ldd < R + Dr || max_pages <= 0 || rows < 0)
     return VLM_ERR_ARG;
@@ -311,34 +320,34 @@ extern "C" int vlm_latent_kv_write(const void* d, long ldd, const void* w, int R
   if (dtype)
     hipLaunchKernelGGL(latent_kv_write_kernel<float>, dim3(rows), dim3(256), 0, st, (const float*)d, ldd, (const float*)w, R, Dr,
                        (const float*)inv_freq, (const int*)tok_seq, (const int*)tok_pos, (const int*)block_table, max_pages,
-                       (float*)pool, eps);
+                       (float*)pool, eps, rot_half);
   else
     hipLaunchKernelGGL(latent_kv_write_kernel<bf16_t>, dim3(rows), dim3(256), 0, st, (const bf16_t*)d, ldd, (const bf16_t*)w, R, Dr,
                        (const float*)inv_freq, (const int*)tok_seq, (const int*)tok_pos, (const int*)block_table, max_pages,
-                       (bf16_t*)pool, eps);
+                       (bf16_t*)pool, eps, rot_half);
   VLM_CHECK_LAUNCH();
   return VLM_OK;
 }
 
 extern "C" int vlm_rope_pairs_rows(const void* q, long ldq, long head_stride, int H, int Dr, const void* inv_freq, const void* tok_pos,
-                                   void* out, long ldo, long out_head_stride, int rows, int dtype, void* stream) {
+                                   void* out, long ldo, long out_head_stride, int rot_half, int rows, int dtype, void* stream) {
   if (!q || !tok_pos || !out || H <= 0 || Dr < 0 || (Dr & 1) || (Dr && !inv_freq) || rows < 0) return VLM_ERR_ARG;
   if (rows == 0 || Dr == 0) return VLM_OK;
   hipStream_t st = (hipStream_t)stream;
   const unsigned nb = (unsigned)(((long)rows * H * (Dr / 2) + 255) / 256);
   if (dtype)
     hipLaunchKernelGGL(rope_pairs_rows_kernel<float>, dim3(nb), dim3(256), 0, st, (const float*)q, ldq, head_stride, H, Dr,
-                       (const float*)inv_freq, (const int*)tok_pos, (float*)out, ldo, out_head_stride, rows);
+                       (const float*)inv_freq, (const int*)tok_pos, (float*)out, ldo, out_head_stride, rows, rot_half);
   else
     hipLaunchKernelGGL(rope_pairs_rows_kernel<bf16_t>, dim3(nb), dim3(256), 0, st, (const bf16_t*)q, ldq, head_stride, H, Dr,
-                       (const float*)inv_freq, (const int*)tok_pos, (float*)out, ldo, out_head_stride, rows);
+                       (const float*)inv_freq, (const int*)tok_pos, (float*)out, ldo, out_head_stride, rows, rot_half);
   VLM_CHECK_LAUNCH();
   return VLM_OK;
 }
 
 extern "C" int vlm_latent_attn(const void* q, const void* pool, const void* tok_seq, const void* tok_pos, const void* block_table,
-                               int max_pages, int H, int R, int Dr, float scale, const void* gate, long ldgate, void* out, int rows,
-                               int dtype, void* stream) {
+                               int max_pages, int H, int R, int Dr, float scale, int window, const void* gate, long ldgate, void* out,
+                               int rows, int dtype, void* stream) {
   if (!q || !pool || !tok_seq || !tok_pos || !block_table || !out || H <= 0 || R <= 0 || Dr < 0 || max_pages <= 0 || rows < 0 ||
       (gate && ldgate < H))
     return VLM_ERR_ARG;
@@ -349,7 +358,7 @@ extern "C" int vlm_latent_attn(const void* q, const void* pool, const void* tok_
   dim3 grid(rows, H);
 #define GO(T, N)                                                                                                                  \
   hipLaunchKernelGGL((latent_attn_kernel<T, N>), grid, dim3(256), lds, st, (const float*)q, (const T*)pool, (const int*)tok_seq,  \
-                     (const int*)tok_pos, (const int*)block_table, max_pages, H, R, Dr, scale, (const T*)gate, ldgate, (float*)out)
+                     (const int*)tok_pos, (const int*)block_table, max_pages, H, R, Dr, scale, window, (const T*)gate, ldgate, (float*)out)
   const int nacc = (R + 255) / 256;
   if (dtype) {
     if (nacc == 1) GO(float, 1); else if (nacc == 2) GO(float, 2); else GO(float, 4);
@@ -363,7 +372,8 @@ extern "C" int vlm_latent_attn(const void* q, const void* pool, const void* tok_
 
 extern "C" int vlm_latent_attn_blocks(const void* q, const void* pool, const void* qb_start, const void* qb_count, int nblocks,
                                       const void* tok_seq, const void* tok_pos, const void* block_table, int max_pages, int H, int R,
-                                      int Dr, float scale, const void* gate, long ldgate, void* out, int dtype, void* stream) {
+                                      int Dr, float scale, int window, const void* gate, long ldgate, void* out, int dtype,
+                                      void* stream) {
   if (!q || !pool || !qb_start || !qb_count || !tok_seq || !tok_pos || !block_table || !out || H <= 0 || R <= 0 || Dr < 0 ||
       max_pages <= 0 || nblocks < 0 || (gate && ldgate < H))
     return VLM_ERR_ARG;
@@ -383,7 +393,7 @@ extern "C" int vlm_latent_attn_blocks(const void* q, const void* pool, const voi
     }                                                                                                                              \
     hipLaunchKernelGGL((latent_attn_block_kernel<T, N>), grid, dim3(256), lds, st, (const float*)q, (const T*)pool,                \
                        (const int*)qb_start, (const int*)qb_count, (const int*)tok_seq, (const int*)tok_pos,                       \
-                       (const int*)block_table, max_pages, H, R, Dr, scale, (const T*)gate, ldgate, (float*)out);                  \
+                       (const int*)block_table, max_pages, H, R, Dr, scale, window, (const T*)gate, ldgate, (float*)out);          \
   } while (0)
   const int nacc = (R + 255) / 256;
   if (dtype) {

@@ -6,6 +6,14 @@
 //
 //   vlm_moe_route        logits fp32 [T][E] -> the `top` largest per token (lowest index wins a tie), softmax over the chosen
 //                        logits only; dense gate table fp32 [T][E] (0 where not chosen) + the chosen (index, weight) lists
+//   vlm_moe_route_scored the same choice with the weights taken from the softmax over ALL experts, times `scale`, not
+//                        renormalised over the chosen ones; and group-limited: the experts form `groups` equal groups of
+//                        neighbours, a group's score is its largest score, and only experts of the `keep` best groups (lowest
+//                        index wins a tie) can be chosen.  groups = keep = 1 is the unrestricted choice.
+//   vlm_glu_rows         out[t][c] = act(g[t][c]) * u[t][c]; act: 0 = tanh-form gelu, 1 = silu, 2 = sigmoid.  With a route table:
+//                        E stacked experts of ff output columns, out[t][e ff + j] = act(g[t][e estride + j]) * u[t][e estride + j]
+//                        * route[t][e] (estride: the distance of two experts' columns in g and u, e.g. 2 ff when every expert's
+//                        gate and up rows lie side by side); T-typed in and out, fp32 inside
 //   vlm_moe_relu2_gate   out[t][c] = relu(up[t][c])^2 * gate[t][c / ff]   for c < E * ff,   relu(up[t][c])^2 for the
 //                        `shared` columns behind them (an expert every token uses); T-typed in and out, fp32 inside
 #include "common.hpp"
@@ -21,13 +29,57 @@ template <> __device__ __forceinline__ void st_f<float>(float* p, float v) { *p 
 template <> __device__ __forceinline__ void st_f<bf16_t>(bf16_t* p, float v) { *p = f2bf(v); }
 
 // one wave per token; lane l owns experts l, l + 64, ... (a bit per owned expert records what earlier rounds took)
-__global__ __launch_bounds__(256) void moe_route_kernel(const float* __restrict__ z, int T, int E, int top, float* __restrict__ gate,
-                                                        int* __restrict__ idx, float* __restrict__ wgt) {
+// scored: weights = softmax over all experts * scale (else: softmax over the chosen logits); groups / keep: see the file head
+__global__ __launch_bounds__(256) void moe_route_kernel(const float* __restrict__ z, int T, int E, int top, int scored, int groups,
+                                                        int keep, float scale, float* __restrict__ gate, int* __restrict__ idx,
+                                                        float* __restrict__ wgt) {
   const int t = blockIdx.x * 4 + (threadIdx.x >> 6), lane = threadIdx.x & 63;
   if (t >= T) return;
   const float* zr = z + (long)t * E;
   for (int e = lane; e < E; e += 64) gate[(long)t * E + e] = 0.f;
-  unsigned taken = 0u;
+  unsigned taken = 0u;                   // bit i: the lane's i-th expert is chosen, or (set before the choice) not eligible
+  float all_max = 0.f, all_den = 1.f;
+  if (scored) {                          // maximum and denominator over ALL experts, fixed order: lane-strided, then the xor tree
+    float m = -INFINITY;
+    for (int e = lane; e < E; e += 64) m = fmaxf(m, zr[e]);
+#pragma unroll
+    for (int o = 32; o > 0; o >>= 1) m = fmaxf(m, __shfl_xor(m, o));
+    float d = 0.f;
+    for (int e = lane; e < E; e += 64) d += expf(zr[e] - m);
+#pragma unroll
+    for (int o = 32; o > 0; o >>= 1) d += __shfl_xor(d, o);
+    all_max = m;
+    all_den = d;
+  }
+  if (groups > 1 && keep < groups) {     // the `keep` groups with the largest member; every other group's experts are marked
+    const int gsz = E / groups;
+    unsigned long long kept = 0ull;      // (groups <= 64)
+    for (int k = 0; k < keep; ++k) {
+      float best = -INFINITY;
+      int bg = 0x7fffffff;
+      for (int e = lane; e < E; e += 64) {
+        const int g = e / gsz;
+        const float v = zr[e];
+        if (!((kept >> g) & 1ull) && (v > best || (v == best && g < bg))) {
+          best = v;
+          bg = g;
+        }
+      }
+#pragma unroll
+      for (int o = 32; o > 0; o >>= 1) {
+        const float ob = __shfl_xor(best, o);
+        const int og = __shfl_xor(bg, o);
+        if (ob > best || (ob == best && og < bg)) {
+          best = ob;
+          bg = og;
+        }
+      }
+      if (bg == 0x7fffffff) break;
+      kept |= 1ull << bg;
+    }
+    for (int e = lane, i = 0; e < E; e += 64, ++i)
+      if (!((kept >> (e / gsz)) & 1ull)) taken |= 1u << i;
+  }
   float zmax = 0.f, denom = 0.f;
   float my_val = 0.f;                    // lane j < top keeps the j-th chosen logit
   int my_idx = -1;
@@ -59,7 +111,7 @@ __global__ __launch_bounds__(256) void moe_route_kernel(const float* __restrict_
     }
     denom += expf(best - zmax);
   }
-  const float w = my_idx >= 0 ? expf(my_val - zmax) / denom : 0.f;
+  const float w = my_idx < 0 ? 0.f : (scored ? expf(my_val - all_max) / all_den * scale : expf(my_val - zmax) / denom);
   if (lane < top) {
     idx[(long)t * top + lane] = my_idx < 0 ? 0 : my_idx;
     wgt[(long)t * top + lane] = w;
@@ -84,14 +136,75 @@ __global__ __launch_bounds__(256) void moe_relu2_gate_kernel(const T* __restrict
   st_f(out + t * ldo + c, u * u * g);
 }
 
+__device__ __forceinline__ float glu_act(float z, int act) {
+  if (act == 0) return 0.5f * z * (1.0f + tanhf(0.7978845608028654f * (z + 0.044715f * z * z * z)));
+  const float sg = 1.f / (1.f + expf(-z));
+  return act == 1 ? z * sg : sg;
+}
+
+template <typename T>
+__global__ __launch_bounds__(256) void glu_rows_kernel(const T* __restrict__ g, long ldg, const T* __restrict__ u, long ldu,
+                                                       const float* __restrict__ route, int E, int ff, int estride, int act,
+                                                       T* __restrict__ out, long ldo, int rows, int dim) {
+  const long i = (long)blockIdx.x * 256 + threadIdx.x;
+  if (i >= (long)rows * dim) return;
+  const long t = i / dim;
+  const int c = (int)(i % dim);
+  float r = 1.f;
+  long cs = c;                            // the column in g and u
+  if (route) {
+    const int e = c / ff;
+    r = route[t * E + e];
+    if (r == 0.f) {                       // an expert the token did not choose: an exact zero whatever its columns hold
+      st_f(out + t * ldo + c, 0.f);
+      return;
+    }
+    cs = (long)e * estride + (c - e * ff);
+  }
+  st_f(out + t * ldo + c, glu_act(ld_f(g + t * ldg + cs), act) * ld_f(u + t * ldu + cs) * r);
+}
+
 }  // namespace
 
 extern "C" int vlm_moe_route(const void* logits, int T, int E, int top, void* gate, void* idx, void* wgt, void* stream) {
   if (!logits || !gate || !idx || !wgt || T < 0 || E <= 0 || top <= 0 || top > E) return VLM_ERR_ARG;
   if (top > 64 || E > 2048) return VLM_ERR_SHAPE;
   if (T == 0) return VLM_OK;
-  hipLaunchKernelGGL(moe_route_kernel, dim3((T + 3) / 4), dim3(256), 0, (hipStream_t)stream, (const float*)logits, T, E, top,
-                     (float*)gate, (int*)idx, (float*)wgt);
+  hipLaunchKernelGGL(moe_route_kernel, dim3((T + 3) / 4), dim3(256), 0, (hipStream_t)stream, (const float*)logits, T, E, top, 0, 1, 1,
+                     1.f, (float*)gate, (int*)idx, (float*)wgt);
+  VLM_CHECK_LAUNCH();
+  return VLM_OK;
+}
+
+extern "C" int vlm_moe_route_scored(const void* logits, int T, int E, int top, int groups, int keep, float scale, void* gate, void* idx,
+                                    void* wgt, void* stream) {
+  if (!logits || !gate || !idx || !wgt || T < 0 || E <= 0 || top <= 0 || top > E || groups <= 0 || keep <= 0 || keep > groups ||
+      E % groups || top > (long)keep * (E / groups))
+    return VLM_ERR_ARG;
+  if (top > 64 || E > 2048 || groups > 64) return VLM_ERR_SHAPE;
+  if (T == 0) return VLM_OK;
+  hipLaunchKernelGGL(moe_route_kernel, dim3((T + 3) / 4), dim3(256), 0, (hipStream_t)stream, (const float*)logits, T, E, top, 1, groups,
+                     keep, scale, (float*)gate, (int*)idx, (float*)wgt);
+  VLM_CHECK_LAUNCH();
+  return VLM_OK;
+}
+
+extern "C" int vlm_glu_rows(const void* g, long ldg, const void* u, long ldu, const void* route, int E, int ff, int estride, int act,
+                            void* out, long ldo, int rows, int dim, int dtype, void* stream) {
+  if (!g || !u || !out || rows < 0 || dim <= 0 || ldo < dim || act < 0 || act > 2) return VLM_ERR_ARG;
+  if (route ? (E <= 0 || ff <= 0 || (long)E * ff != dim || estride < ff || ldg < (long)(E - 1) * estride + ff ||
+               ldu < (long)(E - 1) * estride + ff)
+            : (ldg < dim || ldu < dim))
+    return VLM_ERR_ARG;
+  if (rows == 0) return VLM_OK;
+  const unsigned nb = (unsigned)(((long)rows * dim + 255) / 256);
+  hipStream_t st = (hipStream_t)stream;
+  if (dtype)
+    hipLaunchKernelGGL(glu_rows_kernel<float>, dim3(nb), dim3(256), 0, st, (const float*)g, ldg, (const float*)u, ldu, (const float*)route,
+                       E, ff, estride, act, (float*)out, ldo, rows, dim);
+  else
+    hipLaunchKernelGGL(glu_rows_kernel<bf16_t>, dim3(nb), dim3(256), 0, st, (const bf16_t*)g, ldg, (const bf16_t*)u, ldu,
+                       (const float*)route, E, ff, estride, act, (bf16_t*)out, ldo, rows, dim);
   VLM_CHECK_LAUNCH();
   return VLM_OK;
 }

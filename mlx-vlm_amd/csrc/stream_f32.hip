@@ -15,6 +15,10 @@
 //                              y = (rms(a[t]) * wa + rms(b[t]) * wb) / 2              (two branches side by side, each normed)
 //                              x[t] += rms(y * sigmoid(gate[t] + gate_bias)) * w      and h[t] = T(x[t]) for the next reader
 //   vlm_relu2_rows           out[t][j] = max(in[t][j], 0)^2
+//   vlm_scaled_add_rms       the residual step of a pre-norm sublayer and the norm of the next reader in one pass:
+//                              x[t] += mult * y[t]                                    (y may be NULL: norm only)
+//                              h[t] = x[t] * rsqrt(mean(x[t]^2) + eps) * (w_offset + w)   (w may be NULL: add only; w_offset 1
+//                                                                                      for weights stored around zero)
 #include "common.hpp"
 #include "../../include/vlm_hip.h"
 
@@ -162,6 +166,27 @@ __global__ __launch_bounds__(256) void gated_rms_add_kernel(float* __restrict__ 
 }
 
 template <typename T>
+__global__ __launch_bounds__(256) void scaled_add_rms_kernel(float* __restrict__ x, const T* __restrict__ y, long ldy, float mult,
+                                                             const T* __restrict__ w, float w_offset, T* __restrict__ h, long ldh,
+                                                             int D, float eps) {
+  __shared__ float red[4];
+  const long t = blockIdx.x;
+  float* xr = x + t * D;
+  float q = 0.f;
+  for (int d = threadIdx.x; d < D; d += 256) {          // (every lane re-reads only the entries it wrote)
+    float v = xr[d];
+    if (y) {
+      v = fmaf(mult, ld_f(y + t * ldy + d), v);
+      xr[d] = v;
+    }
+    q += v * v;
+  }
+  if (!w) return;
+  const float r = 1.0f / sqrtf(block_sum(q, red) / (float)D + eps);
+  for (int d = threadIdx.x; d < D; d += 256) st_f(h + t * ldh + d, xr[d] * r * (w_offset + ld_f(w + d)));
+}
+
+template <typename T>
 __global__ __launch_bounds__(256) void relu2_rows_kernel(const T* __restrict__ in, long ldi, T* __restrict__ out, long ldo, int rows,
                                                          int dim) {
   const long i = (long)blockIdx.x * 256 + threadIdx.x;
@@ -280,6 +305,17 @@ extern "C" int vlm_relu2_rows(const void* in, long ldi, void* out, long ldo, int
   const unsigned nb = (unsigned)(((long)rows * dim + 255) / 256);
   if (dtype) hipLaunchKernelGGL(relu2_rows_kernel<float>, dim3(nb), dim3(256), 0, st, (const float*)in, ldi, (float*)out, ldo, rows, dim);
   else hipLaunchKernelGGL(relu2_rows_kernel<bf16_t>, dim3(nb), dim3(256), 0, st, (const bf16_t*)in, ldi, (bf16_t*)out, ldo, rows, dim);
+  VLM_CHECK_LAUNCH();
+  return VLM_OK;
+}
+
+extern "C" int vlm_scaled_add_rms(void* x, const void* y, long ldy, float mult, const void* w, float w_offset, void* h, long ldh, int rows,
+                                  int D, float eps, int dtype, void* stream) {
+  if (!x || !STREAM_ARGS_OK(rows, D) || (y && ldy < D) || (!y && !w) || (w && (!h || ldh < D))) return VLM_ERR_ARG;
+  if (rows == 0) return VLM_OK;
+  hipStream_t st = (hipStream_t)stream;
+  if (dtype) hipLaunchKernelGGL(scaled_add_rms_kernel<float>, dim3(rows), dim3(256), 0, st, (float*)x, (const float*)y, ldy, mult, (const float*)w, w_offset, (float*)h, ldh, D, eps);
+  else hipLaunchKernelGGL(scaled_add_rms_kernel<bf16_t>, dim3(rows), dim3(256), 0, st, (float*)x, (const bf16_t*)y, ldy, mult, (const bf16_t*)w, w_offset, (bf16_t*)h, ldh, D, eps);
   VLM_CHECK_LAUNCH();
   return VLM_OK;
 }

@@ -3,13 +3,18 @@
 // and an elementwise sigmoid gate on the output:
 //
 //     s_ij = (q_i . k_j) * scale * temp[h]        j visible from i  <=>  0 <= i - j < window  (window <= 0: every j <= i)
-//     o_i  = sum_j softmax_j(s_ij) v_j * sigmoid(gate_i)
+//     s_ij <- cap * tanh(s_ij / cap)              when a score cap is given (cap > 0)
+//     o_i  = sum_j softmax_j(s_ij) v_j * sigmoid(gate_i)        gate_i: one number per value column, or one per head
 //
 //   vlm_headnorm_rope_rows   x rows [T][heads][D] (T-typed) -> RMS norm per head (weight [D] shared by the heads, may be NULL)
 //                            -> rotation of the pairs (2 i, 2 i + 1), i < rot_dims / 2, by pos * inv_freq[i] -> fp32, either
 //                            dense [T][heads][D] (queries) or into the paged pool [page][64][heads * D] of the token's sequence
 //                            (keys).  raw_pool (T-typed, same paging): the rows as they came, for designs whose values are the
-//                            un-normed, un-rotated keys (or any separately projected value rows).
+//                            un-normed, un-rotated keys.
+//   vlm_headnorm_rows        the same pass from an argument block, with what further designs need: a bias added to the rows
+//                            first, an RMS norm WITHOUT a weight, a multiplier that grows with the logarithm of the position
+//                            (1 + coef * ln(floor((pos + 1) / every) + 1), for queries), and separately projected value rows
+//                            [T][heads][Dv] (+ bias) copied into their own paged pool in the same launch.
 //   vlm_window_attn_blocks   prompt form: workgroup = (block of up to 16 consecutive queries of one sequence, head); tiles of 16
 //                            keys at multiples of 16 counted from the sequence's first token go through LDS once per block, and
 //                            every query runs the same per-tile update in the same order whatever block it sits in (a tile with
@@ -27,32 +32,39 @@ namespace {
 constexpr int PAGE = 64;
 constexpr int QB = 16, KT = 16;
 
-// grid (tokens, heads), one wave
+__device__ __forceinline__ float capped(float s, float cap) { return cap > 0.f ? cap * tanhf(s / cap) : s; }
+
+// grid (tokens, heads), one wave.  norm: 0 = none, 1 = RMS norm (times w when given)
 template <typename T>
-__global__ __launch_bounds__(64) void headnorm_rope_kernel(const T* __restrict__ x, long ldx, int D, const T* __restrict__ w, float eps,
-                                                           int rot_dims, const float* __restrict__ inv_freq,
+__global__ __launch_bounds__(64) void headnorm_rope_kernel(const T* __restrict__ x, long ldx, int D, const T* __restrict__ bias,
+                                                           const T* __restrict__ w, int norm, float eps, int rot_dims,
+                                                           const float* __restrict__ inv_freq, float temp_coef, int temp_every,
                                                            const int* __restrict__ tok_pos, const int* __restrict__ tok_seq,
                                                            const int* __restrict__ block_table, int max_pages,
-                                                           float* __restrict__ out, T* __restrict__ raw_pool) {
+                                                           float* __restrict__ out, const T* __restrict__ raw, long ldraw, int Draw,
+                                                           const T* __restrict__ raw_bias, T* __restrict__ raw_pool) {
   const long t = blockIdx.x;
   const int h = blockIdx.y, nh = gridDim.y, lane = threadIdx.x;
   const T* src = x + t * ldx + (long)h * D;
+  const T* bs = bias ? bias + (long)h * D : nullptr;
   const int pos = tok_pos[t];
   long row = t;                                          // dense output row, or the token's place in the pool
   if (block_table) row = (long)block_table[(long)tok_seq[t] * max_pages + pos / PAGE] * PAGE + pos % PAGE;
   float* dst = out + (row * nh + h) * D;
   float ss = 0.f;
   for (int i = lane; i < D; i += 64) {
-    const float v = ld_f(src + i);
+    const float v = ld_f(src + i) + (bs ? ld_f(bs + i) : 0.f);
     ss += v * v;
   }
 #pragma unroll
   for (int o = 32; o > 0; o >>= 1) ss += __shfl_xor(ss, o);
-  const float r = w ? 1.0f / sqrtf(ss / (float)D + eps) : 1.f;
+  float r = norm ? 1.0f / sqrtf(ss / (float)D + eps) : 1.f;
+  // (the multiplier is applied to the normed value as one more factor, so a design without it keeps its bits)
+  const float mult = temp_every > 0 ? 1.f + temp_coef * logf((float)((pos + 1) / temp_every) + 1.f) : 1.f;
   for (int i = lane; i < D / 2 + (D & 1); i += 64) {     // one pair per lane and trip (an odd last dimension passes alone)
     const int i0 = 2 * i, i1 = 2 * i + 1;
-    float u = ld_f(src + i0) * r * (w ? ld_f(w + i0) : 1.f);
-    float v = i1 < D ? ld_f(src + i1) * r * (w ? ld_f(w + i1) : 1.f) : 0.f;
+    float u = (ld_f(src + i0) + (bs ? ld_f(bs + i0) : 0.f)) * r * (w ? ld_f(w + i0) : 1.f);
+    float v = i1 < D ? (ld_f(src + i1) + (bs ? ld_f(bs + i1) : 0.f)) * r * (w ? ld_f(w + i1) : 1.f) : 0.f;
     if (i1 < rot_dims) {
       float sn, cs;
       sincosf((float)pos * inv_freq[i], &sn, &cs);
@@ -60,12 +72,21 @@ __global__ __launch_bounds__(64) void headnorm_rope_kernel(const T* __restrict__
       v = v * cs + u * sn;
       u = u2;
     }
+    if (temp_every > 0) {
+      u *= mult;
+      v *= mult;
+    }
     dst[i0] = u;
     if (i1 < D) dst[i1] = v;
   }
   if (raw_pool) {
-    T* rd = raw_pool + (row * nh + h) * D;
-    for (int i = lane; i < D; i += 64) rd[i] = src[i];
+    T* rd = raw_pool + (row * nh + h) * Draw;
+    const T* rs = raw + t * ldraw + (long)h * Draw;
+    if (raw_bias) {
+      for (int i = lane; i < Draw; i += 64) st_f(rd + i, ld_f(rs + i) + ld_f(raw_bias + (long)h * Draw + i));
+    } else {
+      for (int i = lane; i < Draw; i += 64) rd[i] = rs[i];
+    }
   }
 }
 
@@ -76,8 +97,8 @@ __global__ __launch_bounds__(256) void window_attn_block_kernel(const float* __r
                                                                 const int* __restrict__ qb_count, const int* __restrict__ tok_seq,
                                                                 const int* __restrict__ tok_pos, const int* __restrict__ block_table,
                                                                 int max_pages, int H, int KH, int D, int Dv, float scale,
-                                                                const T* __restrict__ temp, int window, const T* __restrict__ gate,
-                                                                long ldgate, T* __restrict__ out, long ldo) {
+                                                                const T* __restrict__ temp, int window, float cap, const T* __restrict__ gate,
+                                                                long ldgate, int gate_head, T* __restrict__ out, long ldo) {
   extern __shared__ __align__(16) float smem[];
   const int DP = (D + 3) & ~3, KP = DP + 4, VP = NACC * 16;
   float* qs = smem;                         // [QB][DP]
@@ -134,7 +155,7 @@ __global__ __launch_bounds__(256) void window_attn_block_kernel(const float* __r
       }
       const int dist = pos0 + r16 - (j0 + l16);
       const bool seen = r16 < nq && dist >= 0 && (window <= 0 || dist < window);
-      ps[r16 * (KT + 1) + l16] = seen ? d * sc : -INFINITY;
+      ps[r16 * (KT + 1) + l16] = seen ? capped(d * sc, cap) : -INFINITY;
     }
     __syncthreads();
     if (tid < QB) {                         // per query: running maximum, tile weights, running sum (fixed order over the tile)
@@ -177,7 +198,7 @@ __global__ __launch_bounds__(256) void window_attn_block_kernel(const float* __r
       const int c = l16 + 16 * b;
       if (c < Dv) {
         float o = acc[b] * inv;
-        if (gate) o *= 1.f / (1.f + expf(-ld_f(gate + t * ldgate + (long)h * Dv + c)));
+        if (gate) o *= 1.f / (1.f + expf(-ld_f(gate + t * ldgate + (gate_head ? (long)h : (long)h * Dv + c))));
         st_f(out + t * ldo + (long)h * Dv + c, o);
       }
     }
@@ -190,8 +211,8 @@ __global__ __launch_bounds__(256) void window_attn_row_kernel(const float* __res
                                                               const T* __restrict__ vpool, const int* __restrict__ tok_seq,
                                                               const int* __restrict__ tok_pos, const int* __restrict__ block_table,
                                                               int max_pages, int H, int KH, int D, int Dv, float scale,
-                                                              const T* __restrict__ temp, int window, const T* __restrict__ gate,
-                                                              long ldgate, T* __restrict__ out, long ldo) {
+                                                              const T* __restrict__ temp, int window, float cap, const T* __restrict__ gate,
+                                                              long ldgate, int gate_head, T* __restrict__ out, long ldo) {
   extern __shared__ __align__(16) float smem[];
   float* qs = smem;              // [D]
   float* ps = qs + ((D + 3) & ~3);  // [256]
@@ -216,7 +237,7 @@ __global__ __launch_bounds__(256) void window_attn_row_kernel(const float* __res
       const float* kr = kpool + (((long)bt[j / PAGE] * PAGE + j % PAGE) * KH + kh) * D;
       float d = 0.f;
       for (int i = 0; i < D; ++i) d = fmaf(qs[i], kr[i], d);
-      s = d * sc;
+      s = capped(d * sc, cap);
     }
     float mx = s;
 #pragma unroll
@@ -255,7 +276,7 @@ __global__ __launch_bounds__(256) void window_attn_row_kernel(const float* __res
     const int c = tid + a * 256;
     if (c < Dv) {
       float o = acc[a] * inv;
-      if (gate) o *= 1.f / (1.f + expf(-ld_f(gate + t * ldgate + (long)h * Dv + c)));
+      if (gate) o *= 1.f / (1.f + expf(-ld_f(gate + t * ldgate + (gate_head ? (long)h : (long)h * Dv + c))));
       st_f(out + t * ldo + (long)h * Dv + c, o);
     }
   }
@@ -283,8 +304,8 @@ __global__ __launch_bounds__(256) void window_attn_row_vec_kernel(const float* _
                                                                   const T* __restrict__ vpool, const int* __restrict__ tok_seq,
                                                                   const int* __restrict__ tok_pos, const int* __restrict__ block_table,
                                                                   int max_pages, int H, int KH, int D, int Dv, float scale,
-                                                                  const T* __restrict__ temp, int window, const T* __restrict__ gate,
-                                                                  long ldgate, T* __restrict__ out, long ldo) {
+                                                                  const T* __restrict__ temp, int window, float cap, const T* __restrict__ gate,
+                                                                  long ldgate, int gate_head, T* __restrict__ out, long ldo) {
   extern __shared__ __align__(16) float smem[];
   float* qs = smem;                  // [D]
   float* sc = qs + D;                // [KC] scores, then weights
@@ -328,7 +349,7 @@ __global__ __launch_bounds__(256) void window_attn_row_vec_kernel(const float* _
       }
       d += vlm_dpp<0xB1, 0xf>(0.f, d);     // quad_perm [1,0,3,2]
       d += vlm_dpp<0x4E, 0xf>(0.f, d);     // quad_perm [2,3,0,1]
-      if (qp == 0 && j < nk) sc[j] = d * scl;
+      if (qp == 0 && j < nk) sc[j] = capped(d * scl, cap);
     }
     __syncthreads();
     float mx = -INFINITY;
@@ -371,42 +392,58 @@ __global__ __launch_bounds__(256) void window_attn_row_vec_kernel(const float* _
     float o = 0.f;
     for (int pp = 0; pp < nparts; ++pp) o += part[(pp * ngroups + c / 8) * 8 + (c & 7)];
     o *= inv;
-    if (gate) o *= 1.f / (1.f + expf(-ld_f(gate + t * ldgate + (long)h * Dv + c)));
+    if (gate) o *= 1.f / (1.f + expf(-ld_f(gate + t * ldgate + (gate_head ? (long)h : (long)h * Dv + c))));
     st_f(out + t * ldo + (long)h * Dv + c, o);
   }
 }
 
 }  // namespace
 
-extern "C" int vlm_headnorm_rope_rows(const void* x, long ldx, int heads, int D, const void* w, float eps, int rot_dims,
-                                      const void* inv_freq, const void* tok_pos, const void* tok_seq, const void* block_table,
-                                      int max_pages, void* out, void* raw_pool, int rows, int dtype, void* stream) {
-  if (!x || !tok_pos || !out || heads <= 0 || D <= 0 || rot_dims < 0 || rot_dims > D || (rot_dims & 1) || (rot_dims && !inv_freq) ||
-      ldx < (long)heads * D || rows < 0 || (block_table && (!tok_seq || max_pages <= 0)) || (raw_pool && !block_table))
+static int headnorm_launch(const vlm_headnorm_args* a, int rows, int dtype, void* stream) {
+  if (!a || !a->x || !a->tok_pos || !a->out || a->heads <= 0 || a->D <= 0 || a->rot_dims < 0 || a->rot_dims > a->D || (a->rot_dims & 1) ||
+      (a->rot_dims && !a->inv_freq) || a->ldx < (long)a->heads * a->D || rows < 0 || (a->block_table && (!a->tok_seq || a->max_pages <= 0)) ||
+      (a->raw_pool && (!a->block_table || !a->raw || a->Draw <= 0 || a->ldraw < (long)a->heads * a->Draw)) || (a->raw_bias && !a->raw_pool))
     return VLM_ERR_ARG;
   if (rows == 0) return VLM_OK;
-  if (heads > 65535) return VLM_ERR_SHAPE;
+  if (a->heads > 65535) return VLM_ERR_SHAPE;
   hipStream_t st = (hipStream_t)stream;
   if (dtype)
-    hipLaunchKernelGGL(headnorm_rope_kernel<float>, dim3(rows, heads), dim3(64), 0, st, (const float*)x, ldx, D, (const float*)w, eps,
-                       rot_dims, (const float*)inv_freq, (const int*)tok_pos, (const int*)tok_seq, (const int*)block_table, max_pages,
-                       (float*)out, (float*)raw_pool);
+    hipLaunchKernelGGL(headnorm_rope_kernel<float>, dim3(rows, a->heads), dim3(64), 0, st, (const float*)a->x, a->ldx, a->D,
+                       (const float*)a->bias, (const float*)a->w, a->norm, a->eps, a->rot_dims, a->inv_freq, a->temp_coef, a->temp_every,
+                       a->tok_pos, a->tok_seq, a->block_table, a->max_pages, a->out, (const float*)a->raw, a->ldraw, a->Draw,
+                       (const float*)a->raw_bias, (float*)a->raw_pool);
   else
-    hipLaunchKernelGGL(headnorm_rope_kernel<bf16_t>, dim3(rows, heads), dim3(64), 0, st, (const bf16_t*)x, ldx, D, (const bf16_t*)w, eps,
-                       rot_dims, (const float*)inv_freq, (const int*)tok_pos, (const int*)tok_seq, (const int*)block_table, max_pages,
-                       (float*)out, (bf16_t*)raw_pool);
+    hipLaunchKernelGGL(headnorm_rope_kernel<bf16_t>, dim3(rows, a->heads), dim3(64), 0, st, (const bf16_t*)a->x, a->ldx, a->D,
+                       (const bf16_t*)a->bias, (const bf16_t*)a->w, a->norm, a->eps, a->rot_dims, a->inv_freq, a->temp_coef, a->temp_every,
+                       a->tok_pos, a->tok_seq, a->block_table, a->max_pages, a->out, (const bf16_t*)a->raw, a->ldraw, a->Draw,
+                       (const bf16_t*)a->raw_bias, (bf16_t*)a->raw_pool);
   VLM_CHECK_LAUNCH();
   return VLM_OK;
 }
 
+extern "C" int vlm_headnorm_rows(const vlm_headnorm_args* a, int rows, int dtype, void* stream) {
+  return headnorm_launch(a, rows, dtype, stream);
+}
+
+extern "C" int vlm_headnorm_rope_rows(const void* x, long ldx, int heads, int D, const void* w, float eps, int rot_dims,
+                                      const void* inv_freq, const void* tok_pos, const void* tok_seq, const void* block_table,
+                                      int max_pages, void* out, void* raw_pool, int rows, int dtype, void* stream) {
+  vlm_headnorm_args a = {};
+  a.x = x; a.ldx = ldx; a.heads = heads; a.D = D; a.w = w; a.norm = w != nullptr; a.eps = eps; a.rot_dims = rot_dims;
+  a.inv_freq = (const float*)inv_freq; a.tok_pos = (const int*)tok_pos; a.tok_seq = (const int*)tok_seq;
+  a.block_table = (const int*)block_table; a.max_pages = max_pages; a.out = (float*)out;
+  if (raw_pool) { a.raw = x; a.ldraw = ldx; a.Draw = D; a.raw_pool = raw_pool; }       // the rows as they came
+  return headnorm_launch(&a, rows, dtype, stream);
+}
+
 #define WINDOW_ARGS_BAD                                                                                                             \
   (!q || !kpool || !vpool || !tok_seq || !tok_pos || !block_table || !out || H <= 0 || KH <= 0 || H % KH || D <= 0 || Dv <= 0 ||      \
-   max_pages <= 0 || (gate && ldgate < (long)H * Dv) || ldo < (long)H * Dv)
+   max_pages <= 0 || (gate && ldgate < (gate_head ? (long)H : (long)H * Dv)) || ldo < (long)H * Dv || !(cap >= 0.f))
 
 extern "C" int vlm_window_attn_blocks(const void* q, const void* kpool, const void* vpool, const void* qb_start, const void* qb_count,
                                       int nblocks, const void* tok_seq, const void* tok_pos, const void* block_table, int max_pages,
-                                      int H, int KH, int D, int Dv, float scale, const void* temp, int window, const void* gate,
-                                      long ldgate, void* out, long ldo, int dtype, void* stream) {
+                                      int H, int KH, int D, int Dv, float scale, const void* temp, int window, float cap,
+                                      const void* gate, long ldgate, int gate_head, void* out, long ldo, int dtype, void* stream) {
   if (WINDOW_ARGS_BAD || !qb_start || !qb_count || nblocks < 0) return VLM_ERR_ARG;
   if (nblocks == 0) return VLM_OK;
   const int nacc = (Dv + 15) / 16 <= 4 ? 4 : ((Dv + 15) / 16 <= 8 ? 8 : 16);
@@ -418,7 +455,7 @@ extern "C" int vlm_window_attn_blocks(const void* q, const void* kpool, const vo
 #define GO(T, N)                                                                                                                    \
   hipLaunchKernelGGL((window_attn_block_kernel<T, N>), grid, dim3(256), lds, st, (const float*)q, (const float*)kpool, (const T*)vpool, \
                      (const int*)qb_start, (const int*)qb_count, (const int*)tok_seq, (const int*)tok_pos, (const int*)block_table,  \
-                     max_pages, H, KH, D, Dv, scale, (const T*)temp, window, (const T*)gate, ldgate, (T*)out, ldo)
+                     max_pages, H, KH, D, Dv, scale, (const T*)temp, window, cap, (const T*)gate, ldgate, gate_head, (T*)out, ldo)
   if (dtype) {
     if (nacc == 4) GO(float, 4); else if (nacc == 8) GO(float, 8); else GO(float, 16);
   } else {
@@ -431,8 +468,8 @@ extern "C" int vlm_window_attn_blocks(const void* q, const void* kpool, const vo
 
 extern "C" int vlm_window_attn_rows(const void* q, const void* kpool, const void* vpool, const void* tok_seq, const void* tok_pos,
                                     const void* block_table, int max_pages, int H, int KH, int D, int Dv, float scale,
-                                    const void* temp, int window, const void* gate, long ldgate, void* out, long ldo, int rows,
-                                    int dtype, void* stream) {
+                                    const void* temp, int window, float cap, const void* gate, long ldgate, int gate_head, void* out,
+                                    long ldo, int rows, int dtype, void* stream) {
   if (WINDOW_ARGS_BAD || rows < 0) return VLM_ERR_ARG;
   if (rows == 0) return VLM_OK;
   if (Dv > 1024 || D > 8192 || H > 65535) return VLM_ERR_SHAPE;
@@ -443,11 +480,11 @@ extern "C" int vlm_window_attn_rows(const void* q, const void* kpool, const void
     if (dtype)
       hipLaunchKernelGGL(window_attn_row_vec_kernel<float>, grid, dim3(256), ldsv, st, (const float*)q, (const float*)kpool,
                          (const float*)vpool, (const int*)tok_seq, (const int*)tok_pos, (const int*)block_table, max_pages, H, KH, D, Dv,
-                         scale, (const float*)temp, window, (const float*)gate, ldgate, (float*)out, ldo);
+                         scale, (const float*)temp, window, cap, (const float*)gate, ldgate, gate_head, (float*)out, ldo);
     else
       hipLaunchKernelGGL(window_attn_row_vec_kernel<bf16_t>, grid, dim3(256), ldsv, st, (const float*)q, (const float*)kpool,
                          (const bf16_t*)vpool, (const int*)tok_seq, (const int*)tok_pos, (const int*)block_table, max_pages, H, KH, D,
-                         Dv, scale, (const bf16_t*)temp, window, (const bf16_t*)gate, ldgate, (bf16_t*)out, ldo);
+                         Dv, scale, (const bf16_t*)temp, window, cap, (const bf16_t*)gate, ldgate, gate_head, (bf16_t*)out, ldo);
     VLM_CHECK_LAUNCH();
     return VLM_OK;
   }
@@ -455,7 +492,7 @@ extern "C" int vlm_window_attn_rows(const void* q, const void* kpool, const void
 #define GO(T, N)                                                                                                                    \
   hipLaunchKernelGGL((window_attn_row_kernel<T, N>), grid, dim3(256), lds, st, (const float*)q, (const float*)kpool, (const T*)vpool, \
                      (const int*)tok_seq, (const int*)tok_pos, (const int*)block_table, max_pages, H, KH, D, Dv, scale,              \
-                     (const T*)temp, window, (const T*)gate, ldgate, (T*)out, ldo)
+                     (const T*)temp, window, cap, (const T*)gate, ldgate, gate_head, (T*)out, ldo)
   const int nacc = (Dv + 255) / 256;
   if (dtype) {
     if (nacc == 1) GO(float, 1); else if (nacc == 2) GO(float, 2); else GO(float, 4);

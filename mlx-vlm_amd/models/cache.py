@@ -693,8 +693,10 @@ class RowCache:
     """Per-layer facade of a layer that caches one row per token (latent attention): the reference's cache attributes that
     make sense for it (`offset`, `state`, `trim`)."""
 
-    def __init__(self, seq: PagedSequence, layer: int):
-        self._seq, self._layer = seq, layer
+    def __init__(self, seq: PagedSequence, layer, shared: bool = False):
+        """layer: the key of the rows in the pool (a layer index, or (layer, name)); shared: the facade of a layer that reads
+        ANOTHER layer's rows - it shows them and never moves the sequence's offset"""
+        self._seq, self._layer, self._shared = seq, layer, shared
 
     @property
     def offset(self):
@@ -711,7 +713,7 @@ class RowCache:
 
     def trim(self, n):
         n = min(self._seq.offset, n)
-        if self._layer == min(self._seq.pool.rows):
+        if not self._shared and self._layer == min(self._seq.pool.rows):
             self._seq.set_offset(self._seq.offset - n)
         return n
 

@@ -642,34 +642,38 @@ def linear_recurrence(args: "_lib.RecurrenceArgs", nseg: int, ntok: int, dtype_f
     check(_lib.lib().vlm_linear_recurrence(C.byref(args), int(nseg), int(ntok), int(bool(dtype_f32)), _stream()), "linear_recurrence")
 
 
-def latent_kv_write(d, w, R, Dr, inv_freq, tok_seq, tok_pos, block_table, pool, eps):
-    """rows of d [T, >= R + Dr] -> (normed latent | rotated key part) at each token's (sequence, position) of the paged pool"""
+def latent_kv_write(d, w, R, Dr, inv_freq, tok_seq, tok_pos, block_table, pool, eps, rot_half=False):
+    """rows of d [T, >= R + Dr] -> (normed latent | rotated key part) at each token's (sequence, position) of the paged pool;
+    rot_half: the rotated pairs are (i, i + Dr / 2) instead of (2 i, 2 i + 1)"""
     _dev(d, w, inv_freq, tok_seq, tok_pos, block_table, pool)
     check(_lib.lib().vlm_latent_kv_write(_p(d), d.stride(0), _p(w), int(R), int(Dr), _p(inv_freq), _p(tok_seq), _p(tok_pos),
-                                         _p(block_table), block_table.shape[1], _p(pool), float(eps), d.shape[0], _f32(d),
-                                         _stream()), "latent_kv_write")
+                                         _p(block_table), block_table.shape[1], _p(pool), float(eps), int(bool(rot_half)), d.shape[0],
+                                         _f32(d), _stream()), "latent_kv_write")
 
 
-def rope_pairs_rows(q, head_stride, H, Dr, inv_freq, tok_pos, out, out_head_stride):
-    """interleaved-pair rotation of a Dr-wide part of every head: q / out are 2-D views at the part's first column"""
+def rope_pairs_rows(q, head_stride, H, Dr, inv_freq, tok_pos, out, out_head_stride, rot_half=False):
+    """rotation of a Dr-wide part of every head (pairs (2 i, 2 i + 1), or (i, i + Dr / 2) with rot_half): q / out are 2-D views
+    at the part's first column"""
     _dev(q, inv_freq, tok_pos, out)
     check(_lib.lib().vlm_rope_pairs_rows(_p(q), q.stride(0), int(head_stride), int(H), int(Dr), _p(inv_freq), _p(tok_pos), _p(out),
-                                         out.stride(0), int(out_head_stride), q.shape[0], _f32(q), _stream()), "rope_pairs_rows")
+                                         out.stride(0), int(out_head_stride), int(bool(rot_half)), q.shape[0], _f32(q), _stream()),
+          "rope_pairs_rows")
 
 
-def latent_attn(q, pool, tok_seq, tok_pos, block_table, H, R, Dr, scale, gate=None, out=None):
-    """q fp32 [T, H, R + Dr] over the latent pool -> fp32 [T, H, R] (times sigmoid(gate[t, h]) when given)"""
+def latent_attn(q, pool, tok_seq, tok_pos, block_table, H, R, Dr, scale, gate=None, out=None, window=0):
+    """q fp32 [T, H, R + Dr] over the latent pool -> fp32 [T, H, R] (times sigmoid(gate[t, h]) when given); window > 0: a query
+    sees itself and the window - 1 tokens before it"""
     _dev(q, pool, tok_seq, tok_pos, block_table, gate, out)
     T = q.shape[0]
     if out is None:
         out = torch.empty(T, H, R, dtype=torch.float32, device=q.device)
     check(_lib.lib().vlm_latent_attn(_p(q), _p(pool), _p(tok_seq), _p(tok_pos), _p(block_table), block_table.shape[1], int(H), int(R),
-                                     int(Dr), float(scale), _p(gate), gate.stride(0) if gate is not None else 0, _p(out), T,
+                                     int(Dr), float(scale), int(window), _p(gate), gate.stride(0) if gate is not None else 0, _p(out), T,
                                      _f32(pool), _stream()), "latent_attn")
     return out
 
 
-def latent_attn_blocks(q, pool, qb_start, qb_count, tok_seq, tok_pos, block_table, H, R, Dr, scale, gate=None, out=None):
+def latent_attn_blocks(q, pool, qb_start, qb_count, tok_seq, tok_pos, block_table, H, R, Dr, scale, gate=None, out=None, window=0):
     """latent_attn over query blocks (qb_start / qb_count int32 [n]: first token and number of consecutive tokens of one
     sequence, at most 16): the prompt form, key tiles staged once per block"""
     _dev(q, pool, qb_start, qb_count, tok_seq, tok_pos, block_table, gate, out)
@@ -677,8 +681,8 @@ def latent_attn_blocks(q, pool, qb_start, qb_count, tok_seq, tok_pos, block_tabl
     if out is None:
         out = torch.empty(T, H, R, dtype=torch.float32, device=q.device)
     check(_lib.lib().vlm_latent_attn_blocks(_p(q), _p(pool), _p(qb_start), _p(qb_count), qb_start.numel(), _p(tok_seq), _p(tok_pos),
-                                            _p(block_table), block_table.shape[1], int(H), int(R), int(Dr), float(scale), _p(gate),
-                                            gate.stride(0) if gate is not None else 0, _p(out), _f32(pool), _stream()),
+                                            _p(block_table), block_table.shape[1], int(H), int(R), int(Dr), float(scale), int(window),
+                                            _p(gate), gate.stride(0) if gate is not None else 0, _p(out), _f32(pool), _stream()),
           "latent_attn_blocks")
     return out
 
@@ -692,6 +696,50 @@ def moe_route(logits, top):
     wgt = torch.empty(T, top, dtype=torch.float32, device=logits.device)
     check(_lib.lib().vlm_moe_route(_p(logits), T, E, int(top), _p(gate), _p(idx), _p(wgt), _stream()), "moe_route")
     return gate, idx, wgt
+
+
+def moe_route_scored(logits, top, groups=1, keep=1, scale=1.0):
+    """moe_route with the weights of the softmax over ALL experts times `scale` (not renormalised), the choice limited to the
+    experts of the `keep` best of `groups` equal groups of neighbours"""
+    _dev(logits)
+    T, E = logits.shape
+    gate = torch.empty(T, E, dtype=torch.float32, device=logits.device)
+    idx = torch.empty(T, top, dtype=torch.int32, device=logits.device)
+    wgt = torch.empty(T, top, dtype=torch.float32, device=logits.device)
+    check(_lib.lib().vlm_moe_route_scored(_p(logits), T, E, int(top), int(groups), int(keep), float(scale), _p(gate), _p(idx), _p(wgt),
+                                          _stream()), "moe_route_scored")
+    return gate, idx, wgt
+
+
+GLU_GELU_TANH, GLU_SILU, GLU_SIGMOID = 0, 1, 2
+
+
+def glu_rows(g, u, act, out=None, route=None, E=0, ff=0, estride=0):
+    """out = act(g) * u over 2-D views with a row pitch (dim: out's columns, else g's); with route (fp32 [T, E]): out [T, E * ff], expert e reads the
+    columns e * estride .. + ff of g and u, times route[t, e]"""
+    _dev(g, u, out, route)
+    rows = g.shape[0]
+    dim = int(E) * int(ff) if route is not None else (out.shape[1] if out is not None else g.shape[1])
+    if out is None:
+        out = torch.empty(rows, dim, dtype=g.dtype, device=g.device)
+    check(_lib.lib().vlm_glu_rows(_p(g), g.stride(0), _p(u), u.stride(0), _p(route), int(E), int(ff), int(estride or ff), int(act),
+                                  _p(out), out.stride(0), rows, dim, _f32(g), _stream()), "glu_rows")
+    return out
+
+
+def scaled_add_rms_(x, y=None, mult=1.0, w=None, w_offset=0.0, eps=1e-6, h=None):
+    """x += mult * y on the fp32 stream (y None: no add); then, with w: h = rms(x) * (w_offset + w) in w's dtype -> h (None
+    without w).  One pass: the residual step of a sublayer and the norm of the next reader."""
+    _dev(x, y, w, h)
+    if x.dtype != torch.float32 or not x.is_contiguous():
+        raise _lib.VlmHipError("scaled_add_rms: contiguous fp32 stream expected")
+    if w is not None and h is None:
+        h = torch.empty(x.shape, dtype=w.dtype, device=x.device)
+    t = y if y is not None else w
+    check(_lib.lib().vlm_scaled_add_rms(_p(x), _p(y), y.stride(0) if y is not None else 0, float(mult), _p(w), float(w_offset), _p(h),
+                                        h.stride(0) if h is not None else 0, x.shape[0], x.shape[1], float(eps), _f32(t), _stream()),
+          "scaled_add_rms")
+    return h
 
 
 def moe_relu2_gate(up, gate, E, ff, shared, out):
@@ -773,22 +821,49 @@ def headnorm_rope_rows(x, heads, D, w, eps, rot_dims, inv_freq, tok_pos, out, to
     return out
 
 
-def window_attn_blocks(q, kpool, vpool, qb_start, qb_count, tok_seq, tok_pos, block_table, H, KH, D, Dv, scale, out, temp=None, window=0,
-                       gate=None):
-    """prompt form of the windowed attention: q fp32 [T, H * D]; out / gate: 2-D views [T, H * Dv] in vpool's dtype"""
-    _dev(q, kpool, vpool, qb_start, qb_count, tok_seq, tok_pos, block_table, out, temp, gate)
-    check(_lib.lib().vlm_window_attn_blocks(_p(q), _p(kpool), _p(vpool), _p(qb_start), _p(qb_count), qb_start.numel(), _p(tok_seq),
-                                            _p(tok_pos), _p(block_table), block_table.shape[1], int(H), int(KH), int(D), int(Dv),
-                                            float(scale), _p(temp), int(window), _p(gate), gate.stride(0) if gate is not None else 0,
-                                            _p(out), out.stride(0), _f32(vpool), _stream()), "window_attn_blocks")
+def headnorm_rows(x, heads, D, tok_pos, out, eps=0.0, norm=True, w=None, bias=None, rot_dims=0, inv_freq=None, temp=None, tok_seq=None,
+                  block_table=None, raw=None, raw_dim=0, raw_bias=None, raw_pool=None):
+    """headnorm_rope_rows with a bias added first, a norm without a weight (norm=True, w=None), a position multiplier
+    temp = (coef, every): 1 + coef * ln(floor((pos + 1) / every) + 1), and value rows `raw` (2-D view [T, heads * raw_dim],
+    + raw_bias) copied into `raw_pool` in the same launch"""
+    _dev(x, w, bias, inv_freq, tok_pos, out, tok_seq, block_table, raw, raw_bias, raw_pool)
+    if out.dtype != torch.float32:
+        raise _lib.VlmHipError("headnorm_rows: fp32 output expected")
+    a = _lib.HeadnormArgs()
+    a.x, a.ldx, a.heads, a.D, a.bias, a.w, a.norm, a.eps = _p(x), x.stride(0), int(heads), int(D), _p(bias), _p(w), int(bool(norm)), float(eps)
+    a.rot_dims, a.inv_freq = int(rot_dims), _p(inv_freq)
+    if temp is not None:
+        a.temp_coef, a.temp_every = float(temp[0]), int(temp[1])
+    a.tok_pos, a.tok_seq, a.block_table = _p(tok_pos), _p(tok_seq), _p(block_table)
+    a.max_pages = block_table.shape[1] if block_table is not None else 0
+    a.out = _p(out)
+    if raw_pool is not None:
+        if raw.dtype != x.dtype or raw_pool.dtype != x.dtype:
+            raise _lib.VlmHipError("headnorm_rows: value rows and their pool have the dtype of x")
+        a.raw, a.ldraw, a.Draw, a.raw_bias, a.raw_pool = _p(raw), raw.stride(0), int(raw_dim), _p(raw_bias), _p(raw_pool)
+    check(_lib.lib().vlm_headnorm_rows(C.byref(a), x.shape[0], _f32(x), _stream()), "headnorm_rows")
     return out
 
 
-def window_attn_rows(q, kpool, vpool, tok_seq, tok_pos, block_table, H, KH, D, Dv, scale, out, temp=None, window=0, gate=None):
+def window_attn_blocks(q, kpool, vpool, qb_start, qb_count, tok_seq, tok_pos, block_table, H, KH, D, Dv, scale, out, temp=None, window=0,
+                       gate=None, cap=0.0, gate_head=False):
+    """prompt form of the windowed attention: q fp32 [T, H * D]; out / gate: 2-D views [T, H * Dv] in vpool's dtype (gate_head:
+    gate [T, H], one number per head); cap > 0: scores pass cap * tanh(. / cap)"""
+    _dev(q, kpool, vpool, qb_start, qb_count, tok_seq, tok_pos, block_table, out, temp, gate)
+    check(_lib.lib().vlm_window_attn_blocks(_p(q), _p(kpool), _p(vpool), _p(qb_start), _p(qb_count), qb_start.numel(), _p(tok_seq),
+                                            _p(tok_pos), _p(block_table), block_table.shape[1], int(H), int(KH), int(D), int(Dv),
+                                            float(scale), _p(temp), int(window), float(cap), _p(gate),
+                                            gate.stride(0) if gate is not None else 0, int(bool(gate_head)), _p(out), out.stride(0),
+                                            _f32(vpool), _stream()), "window_attn_blocks")
+    return out
+
+
+def window_attn_rows(q, kpool, vpool, tok_seq, tok_pos, block_table, H, KH, D, Dv, scale, out, temp=None, window=0, gate=None, cap=0.0,
+                     gate_head=False):
     """decode form of the windowed attention (one workgroup per token and head)"""
     _dev(q, kpool, vpool, tok_seq, tok_pos, block_table, out, temp, gate)
     check(_lib.lib().vlm_window_attn_rows(_p(q), _p(kpool), _p(vpool), _p(tok_seq), _p(tok_pos), _p(block_table), block_table.shape[1],
-                                          int(H), int(KH), int(D), int(Dv), float(scale), _p(temp), int(window), _p(gate),
-                                          gate.stride(0) if gate is not None else 0, _p(out), out.stride(0), q.shape[0], _f32(vpool),
-                                          _stream()), "window_attn_rows")
+                                          int(H), int(KH), int(D), int(Dv), float(scale), _p(temp), int(window), float(cap), _p(gate),
+                                          gate.stride(0) if gate is not None else 0, int(bool(gate_head)), _p(out), out.stride(0),
+                                          q.shape[0], _f32(vpool), _stream()), "window_attn_rows")
     return out
