@@ -123,9 +123,13 @@ class ModelConfig:
             j = lc.kv_from
             if j is None:
                 continue
-            # the source's cache must hold this step's tokens when the layer runs, and be the source's own
-            if not 0 <= j < i or layers[j].type != lc.type or layers[j].kv_from is not None:
-                raise ValueError(f"layer {i}: kv_from must name an earlier {lc.type} layer that has keys and values of its own")
+            # the source's cache must hold this step's tokens when the layer runs: an earlier layer.  A source that itself
+            # reads another layer's cache is followed to the layer that writes it
+            while 0 <= j < i and layers[j].type == lc.type and layers[j].kv_from is not None:
+                j = layers[j].kv_from
+            if not 0 <= j < i or layers[j].type != lc.type:
+                raise ValueError(f"layer {i}: kv_from must name an earlier {lc.type} layer")
+            lc.mixer["kv_from"] = j
             if _cache_sizes(layers[j]) != _cache_sizes(lc):
                 raise ValueError(f"layer {i}: layer {j}, whose cache it reads, has other cache sizes")
         return cls(vocab=int(d["vocab"]), width=int(d["width"]), layers=layers, norm_eps=float(d["norm"]["eps"]),

@@ -40,7 +40,6 @@ class LanguageModel(RaggedLanguageModel):
     # ------------------------------------------------------------------ weights
     def load_weights(self, W: Dict[str, torch.Tensor]):
         cfg, dev, T = self.config, self.device, self.dtype
-        used = set()
 
         def g(name, shape):
             if name not in W:
@@ -48,7 +47,6 @@ class LanguageModel(RaggedLanguageModel):
             t = W[name]
             if tuple(t.shape) != tuple(shape):
                 raise ValueError(f"Tilalorn checkpoint: {name} is {tuple(t.shape)}, the config says {tuple(shape)}")
-            used.add(name)
             return t.to(device=dev, dtype=T).contiguous()
 
         Wd = cfg.width
@@ -102,9 +100,6 @@ class LanguageModel(RaggedLanguageModel):
                     ns.wff, ns.foff = pack_rows([("gate", g(p + "mlp.gate", (ns.ff, Wd))), ("up", g(p + "mlp.up", (ns.ff, Wd)))], T, dev)
                     ns.down = g(p + "mlp.down", (Wd, ns.ff))
             self._L.append(ns)
-        extra = sorted(set(W) - used)
-        if extra:
-            raise ValueError(f"Tilalorn checkpoint: tensors the config does not call for: {extra[:8]}")
         self.pool = HybridPool(len(cfg.layers), rows, {}, self._kv_pool_tokens, self._max_seqs, device=dev, dtype=T)
         return self
 
