@@ -12,10 +12,11 @@
 //   vlm_rope_pairs_rows      rotate the Dr-wide rotary part of every head's query into the fp32 query buffer behind the
 //                            absorbed part
 //                            (both: pairs (2 i, 2 i + 1), or with rot_half the pairs (i, i + Dr / 2))
-//   vlm_latent_attn          causal softmax attention of fp32 queries [T][H][R + Dr] over the pool; key tiles start at
-//                            multiples of 256 counted from the sequence's first token, so the arithmetic of a token does not
-//                            depend on how its prompt was cut; output fp32 [T][H][R], times sigmoid(gate[t][h]) when a gate
-//                            is given
+//   vlm_latent_attn          causal softmax attention of fp32 queries [T][H][R + Dr] over the pool, one workgroup per (token,
+//                            head); output fp32 [T][H][R], times sigmoid(gate[t][h]) when a gate is given.  Rows of whole
+//                            16-byte pieces ((R + Dr) % 8 == 0, R % 8 == 0) are read with 16-byte loads, four lanes to a key;
+//                            other shapes take one key per lane in tiles of 256 keys at multiples of 256 counted from the
+//                            sequence's first token
 // A sliding window (window > 0) limits query i to the keys j with 0 <= i - j < window; tiles still sit at multiples of their
 // size counted from the sequence's first token and start at the tile that holds the window's edge.
 // Scores, softmax and the weighted sum are fp32.  dtype: 0 = bf16, 1 = fp32 for the T-typed pointers.
@@ -307,6 +308,115 @@ __global__ __launch_bounds__(256) void latent_attn_block_kernel(const float* __r
   }
 }
 
+// Decode form for (R + Dr) % 8 == 0 and R % 8 == 0: workgroup = (token, head), the visible keys in chunks of KC rows from the
+// window's edge (or the sequence's first token).
+//   scores : thread (key, quarter): the four lanes of a DPP quad read one cached row in 16-byte pieces (lane q takes pieces q,
+//            q + 4, ...) and add their partial dot products; 64 keys per pass, no barrier between passes;
+//   softmax: chunk maximum and sum over the scores in LDS (online across chunks);
+//   values : thread (group of 8 latent columns, key part): 16-byte loads of the rows' first R columns, a wave covers whole
+//            rows; the key parts' partial sums are added through LDS at the end.
+constexpr int KC = 1024;
+template <typename T>
+__global__ __launch_bounds__(256) void latent_attn_row_vec_kernel(const float* __restrict__ q, const T* __restrict__ pool,
+                                                                  const int* __restrict__ tok_seq, const int* __restrict__ tok_pos,
+                                                                  const int* __restrict__ block_table, int max_pages, int H, int R,
+                                                                  int Dr, float scale, int window, const T* __restrict__ gate,
+                                                                  long ldgate, float* __restrict__ out) {
+  extern __shared__ __align__(16) float smem[];
+  const int Dk = R + Dr;
+  float* qs = smem;                  // [Dk]
+  float* sc = qs + Dk;               // [KC] scores, then weights
+  float* part = sc + KC;             // [256 * 8] partial weighted sums
+  int* rowi = reinterpret_cast<int*>(part + 2048);   // [KC] the chunk's keys as pool rows (page * 64 + place): one table lookup per key
+  __shared__ float red[8];
+  const long t = blockIdx.x;
+  const int h = blockIdx.y, tid = threadIdx.x, wave = tid >> 6;
+  const int pos = tok_pos[t];
+  const int* bt = block_table + (long)tok_seq[t] * max_pages;
+  for (int i = tid; i < Dk; i += 256) qs[i] = q[(t * H + h) * Dk + i];
+  const int ngroups = R / 8, nparts = 256 / ngroups;           // latent-column groups, key parts
+  const int dg = tid % ngroups, kp = tid / ngroups;
+  float acc[8];
+#pragma unroll
+  for (int i = 0; i < 8; ++i) acc[i] = 0.f;
+  float m_run = -INFINITY, l_run = 0.f;
+  const int nkeys = pos + 1;
+  const int first = window > 0 ? max(0, pos - window + 1) : 0;
+  const int D8 = Dk / 8;
+  __syncthreads();
+  for (int k0 = first; k0 < nkeys; k0 += KC) {
+    const int nk = min(KC, nkeys - k0);
+    for (int j = tid; j < nk; j += 256) rowi[j] = bt[(k0 + j) / PAGE] * PAGE + (k0 + j) % PAGE;
+    __syncthreads();
+#pragma unroll 2
+    for (int jb = 0; jb < nk; jb += 64) {
+      const int j = jb + (tid >> 2), qp = tid & 3;
+      float d = 0.f;
+      if (j < nk) {
+        const T* kr = pool + (long)rowi[j] * Dk;
+        for (int c = qp; c < D8; c += 4) {
+          float f[8];
+          load8(kr + c * 8, f);
+          const float4 a = *reinterpret_cast<const float4*>(qs + c * 8), b = *reinterpret_cast<const float4*>(qs + c * 8 + 4);
+          d = fmaf(a.x, f[0], d);
+          d = fmaf(a.y, f[1], d);
+          d = fmaf(a.z, f[2], d);
+          d = fmaf(a.w, f[3], d);
+          d = fmaf(b.x, f[4], d);
+          d = fmaf(b.y, f[5], d);
+          d = fmaf(b.z, f[6], d);
+          d = fmaf(b.w, f[7], d);
+        }
+      }
+      d += vlm_dpp<0xB1, 0xf>(0.f, d);     // quad_perm [1,0,3,2]
+      d += vlm_dpp<0x4E, 0xf>(0.f, d);     // quad_perm [2,3,0,1]
+      if (qp == 0 && j < nk) sc[j] = d * scale;
+    }
+    __syncthreads();
+    float mx = -INFINITY;
+    for (int j = tid; j < nk; j += 256) mx = fmaxf(mx, sc[j]);
+    mx = wave_max(mx);
+    if ((tid & 63) == 0) red[wave] = mx;
+    __syncthreads();
+    const float m_new = fmaxf(m_run, fmaxf(fmaxf(red[0], red[1]), fmaxf(red[2], red[3])));
+    float sum = 0.f;
+    for (int j = tid; j < nk; j += 256) {
+      const float pj = expf(sc[j] - m_new);
+      sc[j] = pj;
+      sum += pj;
+    }
+    sum = wave_sum(sum);
+    if ((tid & 63) == 0) red[4 + wave] = sum;
+    __syncthreads();
+    const float alpha = expf(m_run - m_new);           // (first chunk: exp(-inf) = 0)
+    l_run = l_run * alpha + ((red[4] + red[5]) + (red[6] + red[7]));
+    m_run = m_new;
+#pragma unroll
+    for (int i = 0; i < 8; ++i) acc[i] *= alpha;
+    if (kp < nparts) {
+#pragma unroll 4
+      for (int j = kp; j < nk; j += nparts) {
+        float f[8];
+        load8(pool + (long)rowi[j] * Dk + dg * 8, f);
+        const float pj = sc[j];
+#pragma unroll
+        for (int i = 0; i < 8; ++i) acc[i] = fmaf(pj, f[i], acc[i]);
+      }
+    }
+    __syncthreads();                                    // (the next chunk overwrites sc and red)
+  }
+#pragma unroll
+  for (int i = 0; i < 8; ++i) part[tid * 8 + i] = acc[i];
+  __syncthreads();
+  float gsc = 1.f / l_run;
+  if (gate) gsc *= 1.f / (1.f + expf(-ld_f(gate + t * ldgate + h)));
+  for (int c = tid; c < R; c += 256) {
+    float o = 0.f;
+    for (int pp = 0; pp < nparts; ++pp) o += part[(pp * ngroups + c / 8) * 8 + (c & 7)];
+    out[(t * H + h) * R + c] = o * gsc;
+  }
+}
+
 }  // namespace
 
 extern "C" int vlm_latent_kv_write(const void* d, long ldd, const void* w, int R, int Dr, const void* inv_freq, const void* tok_seq,
@@ -354,8 +464,21 @@ extern "C" int vlm_latent_attn(const void* q, const void* pool, const void* tok_
   if (rows == 0) return VLM_OK;
   if (R > 1024 || H > 65535) return VLM_ERR_SHAPE;
   hipStream_t st = (hipStream_t)stream;
-  const size_t lds = (size_t)(R + Dr + 256 + 8) * sizeof(float);
   dim3 grid(rows, H);
+  if ((R + Dr) % 8 == 0 && R % 8 == 0 && R / 8 <= 256) {
+    const size_t ldsv = (size_t)(R + Dr + 2 * KC + 2048) * sizeof(float);
+    if (dtype)
+      hipLaunchKernelGGL(latent_attn_row_vec_kernel<float>, grid, dim3(256), ldsv, st, (const float*)q, (const float*)pool,
+                         (const int*)tok_seq, (const int*)tok_pos, (const int*)block_table, max_pages, H, R, Dr, scale, window,
+                         (const float*)gate, ldgate, (float*)out);
+    else
+      hipLaunchKernelGGL(latent_attn_row_vec_kernel<bf16_t>, grid, dim3(256), ldsv, st, (const float*)q, (const bf16_t*)pool,
+                         (const int*)tok_seq, (const int*)tok_pos, (const int*)block_table, max_pages, H, R, Dr, scale, window,
+                         (const bf16_t*)gate, ldgate, (float*)out);
+    VLM_CHECK_LAUNCH();
+    return VLM_OK;
+  }
+  const size_t lds = (size_t)(R + Dr + 256 + 8) * sizeof(float);
 #define GO(T, N)                                                                                                                  \
   hipLaunchKernelGGL((latent_attn_kernel<T, N>), grid, dim3(256), lds, st, (const float*)q, (const T*)pool, (const int*)tok_seq,  \
                      (const int*)tok_pos, (const int*)block_table, max_pages, H, R, Dr, scale, window, (const T*)gate, ldgate, (float*)out)
