@@ -272,11 +272,28 @@ def lib():
                 "Build it with `python -c 'import __graft_entry__ as g; g.build()'` or `python mlx-vlm_amd/build.py`.")
         L = C.CDLL(LIB_PATH)
         for name, (res, args) in SIGNATURES.items():
-            fn = getattr(L, name)  # AttributeError if the .so does not export it
+            try:
+                fn = getattr(L, name)  # AttributeError if the .so does not export it
+            except AttributeError:
+                if not PARTIAL:
+                    raise
+                continue               # a partial library: calling an operator it does not hold raises this same error then
             fn.restype = res
             fn.argtypes = args
         _lib = L
     return _lib
+
+
+PARTIAL = False
+
+
+def use_partial_library(path: str):
+    """Point the binding at a library that holds only one model family's operators (build.build(only=...)): must be called
+    before the first operator call.  Operators the library does not export stay unbound and raise AttributeError when called."""
+    global LIB_PATH, PARTIAL
+    if _lib is not None:
+        raise VlmHipError("use_partial_library: the operator library is already loaded")
+    LIB_PATH, PARTIAL = path, True
 
 
 def check(rc: int, what: str = ""):

@@ -58,18 +58,29 @@ def _compile(src: str, force: bool) -> str:
     return obj
 
 
-def build(force: bool = False) -> str:
+def build(force: bool = False, only=None, tag: str = "") -> str:
+    """Compile and link the operator library.  only: source names (without .hip) for a PARTIAL library that holds just the
+    operators one model family needs, linked as lib/libvlm_hip_<tag>.so next to (never in place of) the full library - what the
+    first trace replay of a fresh checkout builds.  Objects are shared between both kinds of build."""
     os.makedirs(LIBDIR, exist_ok=True)
     os.makedirs(OBJDIR, exist_ok=True)
     srcs = sources()
+    lib = LIB
+    if only is not None:
+        want = {os.path.join(CSRC, n + ".hip") for n in only}
+        missing = sorted(want - set(srcs))
+        if missing or not tag:
+            raise ValueError(f"partial build: unknown sources {missing} / no tag")
+        srcs = sorted(want)
+        lib = os.path.join(LIBDIR, f"libvlm_hip_{tag}.so")
     with ThreadPoolExecutor(max_workers=max(1, min(16, os.cpu_count() or 8, len(srcs)))) as ex:
         objs = list(ex.map(lambda s: _compile(s, force), srcs))
-    if force or not os.path.exists(LIB) or any(os.path.getmtime(o) > os.path.getmtime(LIB) for o in objs):
-        cmd = [HIPCC, "--offload-arch=gfx950", "-shared", "-fPIC", "-o", LIB, *objs]
+    if force or not os.path.exists(lib) or any(os.path.getmtime(o) > os.path.getmtime(lib) for o in objs):
+        cmd = [HIPCC, "--offload-arch=gfx950", "-shared", "-fPIC", "-o", lib, *objs]
         r = subprocess.run(cmd, capture_output=True, text=True)
         if r.returncode != 0:
             raise RuntimeError(f"link failed:\n{r.stdout}\n{r.stderr}")
-    return LIB
+    return lib
 
 
 if __name__ == "__main__":

@@ -6,3 +6,6 @@ from .garesun import Model
 from .language import LanguageModel
 
 __all__ = ["Model", "ModelConfig", "LayerConfig", "LanguageModel"]
+
+# the operator sources (csrc/<name>.hip) the model's step function needs: what a trace replay of a fresh checkout compiles
+HIP_SOURCES = ('gemm_bf16', 'gemm256_bf16', 'linear_any', 'stream_f32', 'moe', 'latent_attn', 'linear_recurrence')

@@ -7,3 +7,6 @@ from .language import LanguageModel
 from .luvapel import Model
 
 __all__ = ["Model", "ModelConfig", "LayerConfig", "LanguageModel"]
+
+# the operator sources (csrc/<name>.hip) the model's step function needs: what a trace replay of a fresh checkout compiles
+HIP_SOURCES = ('gemm_bf16', 'gemm256_bf16', 'linear_any', 'stream_f32', 'window_attn', 'delta_rule')

@@ -9,3 +9,6 @@ from .language import LanguageModel
 from .tilalorn import Model
 
 __all__ = ["Model", "ModelConfig", "LayerConfig", "LanguageModel"]
+
+# the operator sources (csrc/<name>.hip) the model's step function needs: what a trace replay of a fresh checkout compiles
+HIP_SOURCES = ('gemm_bf16', 'gemm256_bf16', 'linear_any', 'stream_f32', 'moe', 'latent_attn', 'window_attn')
