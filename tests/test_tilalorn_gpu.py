@@ -186,16 +186,18 @@ def test_latent_attention_windows_both_forms_against_a_dense_softmax(dtype, R, D
 
     Hh = 3
     g = torch.Generator().manual_seed(R)
-    bt = torch.zeros(3, 16, dtype=torch.int32)
-    bt[1, :15] = torch.randperm(15, generator=g).to(torch.int32) + 1
-    pool = (torch.randn(16, PAGE, R + Dr, generator=g) * 0.5).to(dtype)
+    deep = 1890 if R < 100 else 890                     # 1890: the decode form walks more than one chunk of 1024 keys
+    npg = (deep + 37) // PAGE + 2
+    bt = torch.zeros(3, npg, dtype=torch.int32)
+    bt[1, : npg - 1] = torch.randperm(npg - 1, generator=g).to(torch.int32) + 1
+    pool = (torch.randn(npg, PAGE, R + Dr, generator=g) * 0.5).to(dtype)
     tok_seq = torch.tensor([1] * 37 + [2] * 5, dtype=torch.int32)
-    tok_pos = torch.tensor(list(range(890, 927)) + list(range(5)), dtype=torch.int32)
+    tok_pos = torch.tensor(list(range(deep, deep + 37)) + list(range(5)), dtype=torch.int32)
     q = torch.randn(42, Hh, R + Dr, generator=g) * 0.5
     qb_start = torch.tensor([0, 16, 32, 37], dtype=torch.int32).cuda()
     qb_count = torch.tensor([16, 16, 5, 5], dtype=torch.int32).cuda()
     rows = {sq: pool[bt[sq].long()].reshape(-1, R + Dr).double() for sq in (1, 2)}
-    for window in (0, 1, 2, 16, 17, 37, 64, 65, 255, 256, 257, 600):
+    for window in (0, 1, 2, 16, 17, 37, 64, 65, 255, 256, 257, 600, 1024, 1025, 1800):
         want = torch.zeros(42, Hh, R, dtype=F64)
         for t in range(42):
             sq, pos = int(tok_seq[t]), int(tok_pos[t])
