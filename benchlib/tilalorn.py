@@ -16,9 +16,9 @@ def tilalorn_cfg(s, window=1024):
     # the comparison model runs 2 of 8 experts + a shared one of inter / 4 each with two matrices per expert; here an expert has
     # three: 2 of 8 gated experts of inter / 4, or one dense gated layer of inter / 2, are the same work per token
     dense = dict(kind="dense", ff=s["inter"] // 2 // 8 * 8)
-    moe = dict(kind="moe", expert=dict(ff=s["inter"] // 4 // 8 * 8), router=dict(experts=8, top=2, scale=2.5, groups=dict(count=4, keep=2)))
-    att = dict(heads=H, kv_heads=s["kv_heads"], dim=hd, vdim=hd, scale=hd ** -0.5, softcap=50.0, q_temp=dict(coef=0.1, every=1024))
-    lat = dict(heads=H, dim=hd, rot_dim=64, vdim=hd, kv_rank=512, scale=(hd + 64) ** -0.5, rot=dict(base=1000000.0, dims=64), mask=dict(size=window))
+    moe = dict(kind="moe", expert=dict(ff=s["inter"] // 4 // 8 * 8), router=dict(experts=8, top=2, scale=2.0, groups=dict(count=4, keep=2)))
+    att = dict(heads=H, kv_heads=s["kv_heads"], dim=hd, vdim=hd, scale=hd ** -0.5, softcap=30.0, q_temp=dict(coef=0.1, every=1024))
+    lat = dict(heads=H, dim=hd, rot_dim=64, vdim=hd, kv_rank=512, scale=(hd + 64) ** -0.5, rot=dict(base=500000.0, dims=64), mask=dict(size=window))
     pattern = [("attention", att, dense), ("latent_attention", lat, moe), ("latent_attention", lat, dense), ("attention", att, moe),
                ("attention", dict(att, kv_from=3), dense), ("latent_attention", lat, moe)]
     layers = []
@@ -28,7 +28,7 @@ def tilalorn_cfg(s, window=1024):
         if "kv_from" in m:
             m["kv_from"] = i - 1
         layers.append(dict(type=t, mixer=m, mlp=ml))
-    return dict(architecture="Tilalorn", vocab=s["vocab"], width=W, layers=layers, norm=dict(eps=1e-5), residual_mult=0.5)
+    return dict(architecture="Tilalorn", vocab=s["vocab"], width=W, layers=layers, norm=dict(eps=1e-6), residual_mult=0.5)
 
 
 def tilalorn_weights(cfg, dev, seed=0):

@@ -630,8 +630,9 @@ int vlm_latent_attn_blocks(const void* q, const void* pool, const void* qb_start
 
 /* csrc/moe.hip */
 int vlm_moe_route(const void* logits, int T, int E, int top, void* gate, void* idx, void* wgt, void* stream);
-/* ABI v11.  The same choice and outputs with weights = softmax over ALL experts * scale (not renormalised), limited to the experts
- * of the `keep` best of `groups` equal groups of neighbours (a group's score: its largest member; groups <= 64). */
+/* ABI v11.  The same choice and outputs with weights = softmax over ALL experts * scale (no second normalisation), the choice
+ * made among the experts of the `keep` top-ranked of `groups` equally sized blocks of consecutive experts (a block ranks by its
+ * best expert; groups <= 64). */
 int vlm_moe_route_scored(const void* logits, int T, int E, int top, int groups, int keep, float scale, void* gate, void* idx, void* wgt,
                          void* stream);
 /* ABI v11.  out[t][c] = act(g[t][c]) * u[t][c], act 0 = tanh-form gelu, 1 = silu, 2 = sigmoid; with route (fp32 [rows][E]): E stacked

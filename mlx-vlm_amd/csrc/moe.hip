@@ -6,10 +6,10 @@
 //
 //   vlm_moe_route        logits fp32 [T][E] -> the `top` largest per token (lowest index wins a tie), softmax over the chosen
 //                        logits only; dense gate table fp32 [T][E] (0 where not chosen) + the chosen (index, weight) lists
-//   vlm_moe_route_scored the same choice with the weights taken from the softmax over ALL experts, times `scale`, not
-//                        renormalised over the chosen ones; and group-limited: the experts form `groups` equal groups of
-//                        neighbours, a group's score is its largest score, and only experts of the `keep` best groups (lowest
-//                        index wins a tie) can be chosen.  groups = keep = 1 is the unrestricted choice.
+//   vlm_moe_route_scored the same choice with the weights taken from the softmax over ALL experts, times `scale`, with no
+//                        second normalisation over the chosen ones; and group-limited: consecutive experts are cut into
+//                        `groups` blocks of one size, a block ranks by its best expert, and the choice is made among the
+//                        experts of the `keep` top-ranked blocks (lowest index wins a tie).  groups = keep = 1: no limit.
 //   vlm_glu_rows         out[t][c] = act(g[t][c]) * u[t][c]; act: 0 = tanh-form gelu, 1 = silu, 2 = sigmoid.  With a route table:
 //                        E stacked experts of ff output columns, out[t][e ff + j] = act(g[t][e estride + j]) * u[t][e estride + j]
 //                        * route[t][e] (estride: the distance of two experts' columns in g and u, e.g. 2 ff when every expert's
@@ -51,7 +51,7 @@ __global__ __launch_bounds__(256) void moe_route_kernel(const float* __restrict_
     all_max = m;
     all_den = d;
   }
-  if (groups > 1 && keep < groups) {     // the `keep` groups with the largest member; every other group's experts are marked
+  if (groups > 1 && keep < groups) {     // rank the blocks by their best expert, keep `keep` of them; the experts of every other block are marked
     const int gsz = E / groups;
     unsigned long long kept = 0ull;      // (groups <= 64)
     for (int k = 0; k < keep; ++k) {

@@ -18,7 +18,7 @@
 //   vlm_scaled_add_rms       the residual step of a pre-norm sublayer and the norm of the next reader in one pass:
 //                              x[t] += mult * y[t]                                    (y may be NULL: norm only)
 //                              h[t] = x[t] * rsqrt(mean(x[t]^2) + eps) * (w_offset + w)   (w may be NULL: add only; w_offset 1
-//                                                                                      for weights stored around zero)
+//                                                                                      for weights kept as offsets from one)
 #include "common.hpp"
 #include "../../include/vlm_hip.h"
 

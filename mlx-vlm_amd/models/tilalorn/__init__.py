@@ -2,7 +2,7 @@
 (biased projections, unit-RMS queries and keys, a query multiplier that grows with the logarithm of the position, capped
 scores, one sigmoid gate per head; a layer may read an earlier layer's keys and values) or by latent attention with rotary
 positions inside a sliding window (one cached row per token, elementwise sigmoid gate); feed-forwards are dense gated-gelu
-layers or group-limited mixtures of silu experts; tied output head.  Module contract of the other model packages
+layers or group-limited mixtures of silu experts; tied output head.  Same module interface as the other model packages
 (ModelConfig / Model / LanguageModel)."""
 from .config import LayerConfig, ModelConfig
 from .language import LanguageModel

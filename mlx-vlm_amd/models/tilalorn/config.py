@@ -1,5 +1,5 @@
 """config.json of a Tilalorn checkpoint.  Every size and every constant that may differ between checkpoints is read here;
-what the design fixes (activation functions, the rotate-half layout of the rotation, norm weights stored around zero) lives
+what the design fixes (activation functions, the rotate-half layout of the rotation, norm weights kept as offsets from one) lives
 in the model code and the kernels.  Unknown mixer types / feed-forward kinds and inconsistent sizes are refused at load."""
 from __future__ import annotations
 

@@ -1,6 +1,6 @@
 """Tilalorn language model on the HIP operator library (the ragged step of models/ragged.py).
 
-Pre-norm layers on an fp32 residual stream x; norm weights are stored around zero (`rms(x) * (1 + w)`), every sublayer's
+Pre-norm layers on an fp32 residual stream x; a norm weight is kept as its offset from one (`rms(x) * (1 + w)`), every sublayer's
 result enters the stream times one model-wide multiplier m:
     h = norm1(x)        proj = h @ [mixer projections]^T                         one GEMM (rows packed at load)
     attention        : bias + unit RMS per head on q and k (k into the paged fp32 key cache, v + bias into the value cache in

@@ -1,4 +1,4 @@
-"""Model wrapper of a Tilalorn checkpoint: the module contract the generation paths expect from `models.<type>.Model` for a
+"""Model wrapper of a Tilalorn checkpoint: the module interface the generation paths expect from `models.<type>.Model` for a
 text-only model.  The language model keeps its residual stream in fp32 and looks the embedding up inside its step
 (models/ragged.py, TokenIdModel)."""
 from __future__ import annotations

@@ -662,7 +662,7 @@ def rope_pairs_rows(q, head_stride, H, Dr, inv_freq, tok_pos, out, out_head_stri
 
 def latent_attn(q, pool, tok_seq, tok_pos, block_table, H, R, Dr, scale, gate=None, out=None, window=0):
     """q fp32 [T, H, R + Dr] over the latent pool -> fp32 [T, H, R] (times sigmoid(gate[t, h]) when given); window > 0: a query
-    sees itself and the window - 1 tokens before it"""
+    reaches back window - 1 tokens"""
     _dev(q, pool, tok_seq, tok_pos, block_table, gate, out)
     T = q.shape[0]
     if out is None:
@@ -699,8 +699,8 @@ def moe_route(logits, top):
 
 
 def moe_route_scored(logits, top, groups=1, keep=1, scale=1.0):
-    """moe_route with the weights of the softmax over ALL experts times `scale` (not renormalised), the choice limited to the
-    experts of the `keep` best of `groups` equal groups of neighbours"""
+    """moe_route with the weights of the softmax over ALL experts times `scale` (no second normalisation), the choice made among
+    the experts of the `keep` top-ranked of `groups` equally sized blocks of consecutive experts (a block ranks by its best expert)"""
     _dev(logits)
     T, E = logits.shape
     gate = torch.empty(T, E, dtype=torch.float32, device=logits.device)

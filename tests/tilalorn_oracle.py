@@ -94,8 +94,9 @@ def dense_ff(W, p, h):
 
 
 def route(z, r):
-    """router logits z [T, E] -> [T, E] weights: scores = softmax over all experts; only experts of the groups.keep groups with
-    the largest member can be chosen; the `top` best of those get score * scale, the others 0 (lowest index wins a tie)"""
+    """router logits z [T, E] -> [T, E] weights: scores = softmax over all experts; consecutive experts are cut into `count` blocks
+    of one size, a block ranks by its best score, `keep` blocks stay; the `top` best experts inside them get score * scale, every
+    other expert 0 (lowest index wins a tie)"""
     T, E = z.shape
     s = torch.softmax(z, -1)
     g = r.get("groups") or {}
