@@ -117,8 +117,16 @@ class ModelConfig:
     @classmethod
     def from_dict(cls, d: Dict[str, Any]) -> "ModelConfig":
         _need(d, ("vocab", "width", "layers", "norm"), "config")
-        layers = [LayerConfig(type=L["type"], mixer=copy.deepcopy(L["mixer"]), mlp=(copy.deepcopy(L["mlp"]) if L.get("mlp") else None))
-                  for L in d["layers"]]
+        raw = [copy.deepcopy(L["mixer"]) for L in d["layers"]]
+        for i, m in enumerate(raw):
+            # a layer that reads another layer's cache may leave the cache's sizes to that layer's entry
+            j = m.get("kv_from")
+            if j is not None and isinstance(j, int) and 0 <= j < len(raw) and j != i:
+                for k in ("kv_heads", "vdim", "kv_rank", "rot_dim", "rot"):
+                    if k not in m and k in raw[j]:
+                        m[k] = copy.deepcopy(raw[j][k])
+        layers = [LayerConfig(type=L["type"], mixer=m, mlp=(copy.deepcopy(L["mlp"]) if L.get("mlp") else None))
+                  for L, m in zip(d["layers"], raw)]
         for i, lc in enumerate(layers):
             j = lc.kv_from
             if j is None:

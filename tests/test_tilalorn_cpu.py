@@ -29,6 +29,10 @@ def test_config_reads_every_size_and_refuses_what_the_design_does_not_have():
     assert mp.residual_mult == 1.0 and mp.layers[0].mixer["vdim"] == 24          # what an entry leaves out
     chain = ModelConfig.from_dict(H.config([H.attention(), H.attention(kv_from=0), H.latent(), H.attention(kv_from=1)]))
     assert [l.kv_from for l in chain.layers] == [None, 0, None, 0]                # a borrowing source is followed to the owner
+    lean = H.config([H.attention(vdim=40), H.attention(kv_from=0, vdim=40)])
+    del lean["layers"][1]["mixer"]["kv_heads"], lean["layers"][1]["mixer"]["vdim"]      # left to the entry of the layer it reads
+    ml = ModelConfig.from_dict(lean)
+    assert ml.layers[1].mixer["kv_heads"] == 2 and ml.layers[1].mixer["vdim"] == 40
     bad = H.config([H.attention()])
     bad["layers"][0]["type"] = "convolution"
     with pytest.raises(ValueError):
