@@ -583,8 +583,11 @@ int vlm_gelu_tanh_gate_rows(const void* g, long ldg, const void* table, long ldt
 
 /* csrc/linear_recurrence.hip: S_t = a_t S_(t-1) + b_t k_t v_t^T, o_t = S_t^T q_t per head, state fp32 per sequence slot.
  * gated = 0: a = decay[h], b = 1, rotate-half positions on the first rot_dims dimensions of q and k (inv_freq fp32
- * [rot_dims / 2]); gated = 1: exponential gates with a running maximum, normaliser column, denominator (see the file).
- * Then per head: unit RMS (eps), times normw (T [H * Dv], may be NULL), times silu (gate_act 0) or sigmoid (1) of g. */
+ * [rot_dims / 2]); gated = 1: exponential gates with a running maximum, normaliser column, denominator (see the file);
+ * gated = 2 (ABI v12): one forget gate per state row, f = lower + (1 - lower) * sigmoid(k + fbias) with `k` the gate's
+ * pre-activation rows, S <- diag(f) S + (1 - f) v^T (the write key is tied to the gate), q_act 1: q passes silu first.
+ * Then per head: unit RMS (eps), times normw (T [H * Dv], may be NULL), times silu (gate_act 0) or sigmoid (1) of g, or no gate
+ * (gate_act 2, g may be NULL; ABI v12). */
 typedef struct vlm_recurrence_args {
   const void *q, *k, *v, *g;            /* T: row t at + t * ld, head h at + h * D (q, k) / + h * Dv (v, g) */
   long ldq, ldk, ldv, ldg;
@@ -608,6 +611,8 @@ typedef struct vlm_recurrence_args {
   void* out;                            /* T [ntok] rows at ldo */
   long ldo;
   int H, D, Dv, gated;
+  const void *fbias, *lower;            /* gated = 2: T [H * D] each (fbias may be NULL; lower NULL = 0) */
+  int q_act;                            /* gated = 2: 0 = q as projected, 1 = silu(q) */
 } vlm_recurrence_args;
 int vlm_linear_recurrence(const vlm_recurrence_args* a, int nseg, int ntok, int dtype, void* stream);
 
@@ -637,6 +642,14 @@ int vlm_moe_route_scored(const void* logits, int T, int E, int top, int groups, 
                          void* stream);
 /* ABI v11.  out[t][c] = act(g[t][c]) * u[t][c], act 0 = tanh-form gelu, 1 = silu, 2 = sigmoid; with route (fp32 [rows][E]): E stacked
  * experts of ff columns, the columns of expert e in g / u start at e * estride, times route[t][e] (a zero writes an exact zero). */
+/* ABI v12.  Sigmoid-scored routing: s = sigmoid(z); the CHOICE is made on s + correction (fp32 [E] or NULL), among the experts of
+ * the `keep` best of `groups` equally sized blocks of consecutive experts, a block ranking by the sum of its `group_top` largest
+ * choice scores (lowest index wins a tie; the experts of every other block cannot be chosen whatever their score); the weights are
+ * the chosen experts' s (without the correction), divided by their sum + 1e-20 when `normalise`, times scale.  logits: fp32 rows at
+ * ldz >= E + extra; the sigmoid of the `extra` columns behind the experts' goes to extra_out fp32 [T][extra] (gates of experts that
+ * every token uses).  Outputs as vlm_moe_route. */
+int vlm_moe_route_sigmoid(const void* logits, long ldz, int T, int E, int top, int groups, int keep, int group_top, const void* correction,
+                          int normalise, float scale, int extra, void* extra_out, void* gate, void* idx, void* wgt, void* stream);
 int vlm_glu_rows(const void* g, long ldg, const void* u, long ldu, const void* route, int E, int ff, int estride, int act, void* out,
                  long ldo, int rows, int dim, int dtype, void* stream);
 int vlm_moe_relu2_gate(const void* up, long ldu, const void* gate, int E, int ff, int shared, void* out, long ldo, int rows, int dtype,
@@ -652,8 +665,10 @@ int vlm_gated_rms_add(void* x, const void* a, long lda, const void* wa, const vo
 int vlm_relu2_rows(const void* in, long ldi, void* out, long ldo, int rows, int dim, int dtype, void* stream);
 /* ABI v11.  x[t] += mult * y[t] (y T rows at ldy, may be NULL), then h[t] = rms(x[t]) * (w_offset + w) into T rows at ldh (w may be
  * NULL: no norm).  The residual step of a pre-norm sublayer fused with the norm of the next reader. */
-int vlm_scaled_add_rms(void* x, const void* y, long ldy, float mult, const void* w, float w_offset, void* h, long ldh, int rows, int D,
-                       float eps, int dtype, void* stream);
+/* ABI v12: a second addend x[t] += mult2 * y2[t] (y2 may be NULL) in the same pass, and h_f32 = 1: h is written as fp32 rows whatever
+ * T is (a reader that goes on in fp32, e.g. a short convolution over the normed rows). */
+int vlm_scaled_add_rms(void* x, const void* y, long ldy, float mult, const void* y2, long ldy2, float mult2, const void* w, float w_offset,
+                       void* h, long ldh, int h_f32, int rows, int D, float eps, int dtype, void* stream);
 
 /* csrc/delta_rule.hip: delta-rule recurrences (the update reads the old state), state fp32 [slots][H][D][Dv].
  * Prepare passes write fp32 rows; the scan + finish take them.  Segments as in vlm_linear_recurrence. */
@@ -709,7 +724,8 @@ int vlm_delta_rule(const vlm_delta_rule_args* a, int nseg, int ntok, int dtype, 
 /* csrc/window_attn.hip: grouped-head softmax attention with a sliding window over paged caches: keys fp32 [pages][64][KH * D]
  * (normed, rotated), values T [pages][64][KH * Dv].  window <= 0: causal without a window.  temp: T [H] or NULL.
  * ABI v11: cap > 0: scores pass cap * tanh(. / cap); gate_head: the gate is one number per head (T [.][H] at ldgate) instead of
- * one per value column. */
+ * one per value column.
+ * ABI v12: sink = 1: the softmax has one more term exp(0) in its denominator, which carries no value. */
 typedef struct vlm_headnorm_args {
   const void* x;                        /* T rows [heads * D] at ldx */
   long ldx;
@@ -730,6 +746,7 @@ typedef struct vlm_headnorm_args {
   int Draw;
   const void* raw_bias;
   void* raw_pool;
+  int rot_half;                         /* ABI v12: 1 = the rotated pairs are (i, i + rot_dims / 2), and the rotation comes BEFORE the norm */
 } vlm_headnorm_args;
 int vlm_headnorm_rows(const vlm_headnorm_args* a, int rows, int dtype, void* stream);
 int vlm_headnorm_rope_rows(const void* x, long ldx, int heads, int D, const void* w, float eps, int rot_dims, const void* inv_freq,
@@ -737,11 +754,52 @@ int vlm_headnorm_rope_rows(const void* x, long ldx, int heads, int D, const void
                            int rows, int dtype, void* stream);
 int vlm_window_attn_blocks(const void* q, const void* kpool, const void* vpool, const void* qb_start, const void* qb_count, int nblocks,
                            const void* tok_seq, const void* tok_pos, const void* block_table, int max_pages, int H, int KH, int D, int Dv,
-                           float scale, const void* temp, int window, float cap, const void* gate, long ldgate, int gate_head, void* out,
-                           long ldo, int dtype, void* stream);
+                           float scale, const void* temp, int window, float cap, int sink, const void* gate, long ldgate, int gate_head,
+                           void* out, long ldo, int dtype, void* stream);
 int vlm_window_attn_rows(const void* q, const void* kpool, const void* vpool, const void* tok_seq, const void* tok_pos,
                          const void* block_table, int max_pages, int H, int KH, int D, int Dv, float scale, const void* temp, int window,
-                         float cap, const void* gate, long ldgate, int gate_head, void* out, long ldo, int rows, int dtype, void* stream);
+                         float cap, int sink, const void* gate, long ldgate, int gate_head, void* out, long ldo, int rows, int dtype,
+                         void* stream);
+
+/* csrc/short_conv.hip (ABI v12): a causal convolution over time on every channel, for the rows of a ragged step:
+ *   out[t][c] = (residual ? in[t][c] : 0) + bias[c] + sum_j w[c][j] * in(t - taps + 1 + j)[c],   then silu when act = 1.
+ * Inputs before the step's first token of a sequence come from the sequence's carry (the last taps - 1 inputs, fp32
+ * [slots][taps - 1][C], oldest first), inputs before position 0 are zero (a slot that is used again needs no clearing).
+ * vlm_short_conv_rows reads the carry; vlm_short_conv_carry, launched after it, moves the carry to the end of the segments. */
+typedef struct vlm_short_conv_args {
+  const void* in;                       /* rows [C] at ldin: fp32 when in_f32, else T */
+  long ldin;
+  int in_f32;
+  const void* w;                        /* T [C][taps], the current token's tap last */
+  const void* bias;                     /* T [C] or NULL */
+  int C, taps, act, residual;
+  float* carry;
+  const int *tok_seq, *tok_pos;         /* [ntok]: the token's sequence slot and position */
+  const int *seg_start, *seg_slot, *seg_pos0;
+  void* out;                            /* rows [C] at ldo: fp32 when out_f32, else T */
+  long ldo;
+  int out_f32;
+} vlm_short_conv_args;
+int vlm_short_conv_rows(const vlm_short_conv_args* a, int ntok, int dtype, void* stream);
+int vlm_short_conv_carry(const vlm_short_conv_args* a, int nseg, int dtype, void* stream);
+
+/* csrc/selective_scan.hip (ABI v12): the selective state-space scan, state fp32 [slots][C][N] carried per sequence:
+ *   dt = softplus(dt_pre + dt_bias)      S[c][n] <- exp(dt_c A[c][n]) S[c][n] + dt_c x_c B_n      A = -exp(A_log)
+ *   y_c = sum_n S[c][n] C_n + D_c x_c    out = y * silu(z)
+ * Segments as in vlm_linear_recurrence; token-by-token arithmetic, so a prompt cut anywhere gives the same bits. */
+typedef struct vlm_selective_scan_args {
+  const void *x, *z;                    /* T rows [C] at ldx / ldz */
+  long ldx, ldz;
+  const float *dt_pre, *B, *Cm;         /* fp32 rows: [C] at lddt, [N] at ldbc each */
+  long lddt, ldbc;
+  const void *dt_bias, *A_log, *D;      /* T [C], T [C][N], T [C] */
+  const int *seg_start, *seg_slot, *seg_pos0;
+  float* state;
+  void* out;                            /* T rows [C] at ldo */
+  long ldo;
+  int C, N;
+} vlm_selective_scan_args;
+int vlm_selective_scan(const vlm_selective_scan_args* a, int nseg, int ntok, int dtype, void* stream);
 
 #ifdef __cplusplus
 }

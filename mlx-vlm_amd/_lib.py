@@ -100,7 +100,7 @@ class RecurrenceArgs(C.Structure):
                    ("kscale", c_float), ("normw", c_void_p), ("gate_act", c_int), ("eps", c_float), ("seg_start", c_void_p),
                    ("seg_slot", c_void_p), ("seg_pos0", c_void_p), ("state", c_void_p), ("mstate", c_void_p), ("mtok", c_void_p),
                    ("mprev", c_void_p), ("raw", c_void_p), ("out", c_void_p), ("ldo", C.c_long), ("H", c_int), ("D", c_int),
-                   ("Dv", c_int), ("gated", c_int)])
+                   ("Dv", c_int), ("gated", c_int), ("fbias", c_void_p), ("lower", c_void_p), ("q_act", c_int)])
 
 
 class DeltaPrepGeneralArgs(C.Structure):
@@ -131,7 +131,23 @@ class HeadnormArgs(C.Structure):
     _fields_ = [("x", c_void_p), ("ldx", C.c_long), ("heads", c_int), ("D", c_int), ("bias", c_void_p), ("w", c_void_p), ("norm", c_int),
                 ("eps", c_float), ("rot_dims", c_int), ("inv_freq", c_void_p), ("temp_coef", c_float), ("temp_every", c_int),
                 ("tok_pos", c_void_p), ("tok_seq", c_void_p), ("block_table", c_void_p), ("max_pages", c_int), ("out", c_void_p),
-                ("raw", c_void_p), ("ldraw", C.c_long), ("Draw", c_int), ("raw_bias", c_void_p), ("raw_pool", c_void_p)]
+                ("raw", c_void_p), ("ldraw", C.c_long), ("Draw", c_int), ("raw_bias", c_void_p), ("raw_pool", c_void_p), ("rot_half", c_int)]
+
+
+class ShortConvArgs(C.Structure):
+    """vlm_short_conv_args (include/vlm_hip.h)"""
+    _fields_ = [("in_", c_void_p), ("ldin", C.c_long), ("in_f32", c_int), ("w", c_void_p), ("bias", c_void_p), ("C", c_int), ("taps", c_int),
+                ("act", c_int), ("residual", c_int), ("carry", c_void_p), ("tok_seq", c_void_p), ("tok_pos", c_void_p),
+                ("seg_start", c_void_p), ("seg_slot", c_void_p), ("seg_pos0", c_void_p), ("out", c_void_p), ("ldo", C.c_long),
+                ("out_f32", c_int)]
+
+
+class SelectiveScanArgs(C.Structure):
+    """vlm_selective_scan_args (include/vlm_hip.h)"""
+    _fields_ = [("x", c_void_p), ("z", c_void_p), ("ldx", C.c_long), ("ldz", C.c_long), ("dt_pre", c_void_p), ("B", c_void_p),
+                ("Cm", c_void_p), ("lddt", C.c_long), ("ldbc", C.c_long), ("dt_bias", c_void_p), ("A_log", c_void_p), ("D", c_void_p),
+                ("seg_start", c_void_p), ("seg_slot", c_void_p), ("seg_pos0", c_void_p), ("state", c_void_p), ("out", c_void_p),
+                ("ldo", C.c_long), ("C", c_int), ("N", c_int)]
 
 
 DECODE_FUSED_TAIL = 1                       # vlm_decode_args.flags
@@ -235,8 +251,13 @@ SIGNATURES = {
     "vlm_moe_route_scored": (c_int, [c_void_p, c_int, c_int, c_int, c_int, c_int, c_float, c_void_p, c_void_p, c_void_p, c_void_p]),
     "vlm_glu_rows": (c_int, [c_void_p, C.c_long, c_void_p, C.c_long, c_void_p, c_int, c_int, c_int, c_int, c_void_p, C.c_long, c_int,
                              c_int, c_int, c_void_p]),
-    "vlm_scaled_add_rms": (c_int, [c_void_p, c_void_p, C.c_long, c_float, c_void_p, c_float, c_void_p, C.c_long, c_int, c_int, c_float,
-                                   c_int, c_void_p]),
+    "vlm_scaled_add_rms": (c_int, [c_void_p, c_void_p, C.c_long, c_float, c_void_p, C.c_long, c_float, c_void_p, c_float, c_void_p, C.c_long,
+                                   c_int, c_int, c_int, c_float, c_int, c_void_p]),
+    "vlm_moe_route_sigmoid": (c_int, [c_void_p, C.c_long, c_int, c_int, c_int, c_int, c_int, c_int, c_void_p, c_int, c_float, c_int,
+                                      c_void_p, c_void_p, c_void_p, c_void_p, c_void_p]),
+    "vlm_short_conv_rows": (c_int, [P(ShortConvArgs), c_int, c_int, c_void_p]),
+    "vlm_short_conv_carry": (c_int, [P(ShortConvArgs), c_int, c_int, c_void_p]),
+    "vlm_selective_scan": (c_int, [P(SelectiveScanArgs), c_int, c_int, c_int, c_void_p]),
     "vlm_headnorm_rows": (c_int, [P(HeadnormArgs), c_int, c_int, c_void_p]),
     "vlm_moe_relu2_gate": (c_int, [c_void_p, C.c_long, c_void_p, c_int, c_int, c_int, c_void_p, C.c_long, c_int, c_int, c_void_p]),
     "vlm_stream_cast": (c_int, [c_void_p, c_void_p, c_int, c_int, c_int, c_void_p]),
@@ -249,9 +270,9 @@ SIGNATURES = {
     "vlm_delta_rule": (c_int, [P(DeltaRuleArgs), c_int, c_int, c_int, c_void_p]),
     "vlm_headnorm_rope_rows": (c_int, [c_void_p, C.c_long, c_int, c_int, c_void_p, c_float, c_int] + [c_void_p] * 4 + [c_int, c_void_p,
                                        c_void_p, c_int, c_int, c_void_p]),
-    "vlm_window_attn_blocks": (c_int, [c_void_p] * 5 + [c_int] + [c_void_p] * 3 + [c_int] * 5 + [c_float, c_void_p, c_int, c_float,
+    "vlm_window_attn_blocks": (c_int, [c_void_p] * 5 + [c_int] + [c_void_p] * 3 + [c_int] * 5 + [c_float, c_void_p, c_int, c_float, c_int,
                                        c_void_p, C.c_long, c_int, c_void_p, C.c_long, c_int, c_void_p]),
-    "vlm_window_attn_rows": (c_int, [c_void_p] * 6 + [c_int] * 5 + [c_float, c_void_p, c_int, c_float, c_void_p, C.c_long, c_int,
+    "vlm_window_attn_rows": (c_int, [c_void_p] * 6 + [c_int] * 5 + [c_float, c_void_p, c_int, c_float, c_int, c_void_p, C.c_long, c_int,
                                      c_void_p, C.c_long, c_int, c_int, c_void_p]),
 }
 

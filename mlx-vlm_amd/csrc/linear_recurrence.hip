@@ -7,7 +7,10 @@
 //   * gated ("mLSTM"): log input gate i_t = cap * tanh((i~ + bias) / cap), log forget gate f_t = logsigmoid(cap * tanh((f~ +
 //     bias) / cap)), running maximum m_t = max(f_t + m_(t-1), i_t) with m_0 = 0, a_t = exp(f_t + m_(t-1) - m_t),
 //     b_t = exp(i_t - m_t); the normaliser n_t = a_t n_(t-1) + b_t k_t rides along as one more COLUMN of S (v extended by a
-//     constant 1), so n_t . q_t is one more output; o_t is divided by max(|n_t . q_t|, exp(-m_t)) + 1e-6.
+//     constant 1), so n_t . q_t is one more output; o_t is divided by max(|n_t . q_t|, exp(-m_t)) + 1e-6;
+//   * gate per state row ("HGRN2"): S_t = diag(f_t) S_(t-1) + (1 - f_t) v_t^T with f_t = lower + (1 - lower) * sigmoid(f~_t + bias)
+//     per head and row - the forget gate is bounded from below and also decides what is written (no separate key); q may pass
+//     silu first.  The gate's pre-activation rows come in through `k`; gate and 1 - gate are evaluated in fp32 on the way into LDS.
 //
 // One kernel serves a whole prompt, a portion of one and a single decoded token: a segment is `len` consecutive tokens of one
 // sequence; its state is read from the sequence's slot (zero when the segment starts at position 0 - a slot that is used
@@ -28,8 +31,9 @@ constexpr int CT = 64;       // state columns per workgroup
 
 __device__ __forceinline__ float logsigmoid_f(float x) { return fminf(x, 0.f) - log1pf(expf(-fabsf(x))); }
 
-template <typename T, bool GATED>
+template <typename T, int MODE>
 __global__ __launch_bounds__(1024) void linear_recurrence_kernel(vlm_recurrence_args p, int P, int TB) {
+  constexpr bool GATED = MODE == 1, ROWGATE = MODE == 2;
   extern __shared__ __align__(16) float smem[];
   const int seg = blockIdx.x, h = blockIdx.y, c0 = blockIdx.z * CT;
   const int D = p.D, Dv = p.Dv, C = Dv + (GATED ? 1 : 0), DP = P * DR;
@@ -40,6 +44,7 @@ __global__ __launch_bounds__(1024) void linear_recurrence_kernel(vlm_recurrence_
   float* vs = ks + TB * DP;               // [TB][CT]
   float* ab = vs + TB * CT;               // [TB][4]: a, b, (gated) i, f / scratch
   float* po = ab + TB * 4;                // [TB][P][CT]
+  float* fs = po + TB * P * CT;           // [TB][DP] (ROWGATE): the forget gate per state row; ks holds 1 - f
   const int t_begin = p.seg_start[seg], t_end = p.seg_start[seg + 1];
   const int slot = p.seg_slot[seg], pos0 = p.seg_pos0[seg];
   const T* q = (const T*)p.q + (long)h * D;
@@ -56,7 +61,7 @@ __global__ __launch_bounds__(1024) void linear_recurrence_kernel(vlm_recurrence_
   //  moved the slot's own value to the end of the segment - every column tile must see the OLD one)
   float m_run = GATED ? p.mprev[(long)seg * p.H + h] : 0.f;
   const int half = p.rot_dims / 2;
-  const float dec = GATED ? 0.f : p.decay[h];
+  const float dec = MODE == 0 ? p.decay[h] : 0.f;
 
   for (int t0 = t_begin; t0 < t_end; t0 += TB) {
     const int nb = min(TB, t_end - t0);
@@ -77,8 +82,18 @@ __global__ __launch_bounds__(1024) void linear_recurrence_kernel(vlm_recurrence_
           qv = i < half ? qv * cs - qo * sn : qv * cs + qo * sn;
           kv = i < half ? kv * cs - ko * sn : kv * cs + ko * sn;
         }
-        qv *= p.qscale;
-        kv *= p.kscale;
+        if (ROWGATE) {
+          if (p.q_act == 1) qv = qv / (1.f + expf(-qv));
+          const float lo = p.lower ? ld_f((const T*)p.lower + (long)h * D + i) : 0.f;
+          const float f = lo + (1.f - lo) / (1.f + expf(-(kv + (p.fbias ? ld_f((const T*)p.fbias + (long)h * D + i) : 0.f))));
+          fs[idx] = f;
+          kv = 1.f - f;
+        } else {
+          qv *= p.qscale;
+          kv *= p.kscale;
+        }
+      } else if (ROWGATE) {
+        fs[idx] = 0.f;
       }
       qs[idx] = qv;
       ks[idx] = kv;
@@ -119,6 +134,21 @@ __global__ __launch_bounds__(1024) void linear_recurrence_kernel(vlm_recurrence_
       const float4* kr = reinterpret_cast<const float4*>(ks + t * DP + row0);
       const float4* qr = reinterpret_cast<const float4*>(qs + t * DP + row0);
       float acc = 0.f;
+      if (ROWGATE) {
+        const float4* fr = reinterpret_cast<const float4*>(fs + t * DP + row0);
+#pragma unroll
+        for (int r = 0; r < DR / 4; ++r) {
+          const float4 kk = kr[r], qq = qr[r], ff = fr[r];
+          s[4 * r + 0] = fmaf(ff.x, s[4 * r + 0], kk.x * bv);
+          acc = fmaf(s[4 * r + 0], qq.x, acc);
+          s[4 * r + 1] = fmaf(ff.y, s[4 * r + 1], kk.y * bv);
+          acc = fmaf(s[4 * r + 1], qq.y, acc);
+          s[4 * r + 2] = fmaf(ff.z, s[4 * r + 2], kk.z * bv);
+          acc = fmaf(s[4 * r + 2], qq.z, acc);
+          s[4 * r + 3] = fmaf(ff.w, s[4 * r + 3], kk.w * bv);
+          acc = fmaf(s[4 * r + 3], qq.w, acc);
+        }
+      } else
 #pragma unroll
       for (int r = 0; r < DR / 4; ++r) {
         const float4 kk = kr[r], qq = qr[r];
@@ -186,12 +216,12 @@ __global__ __launch_bounds__(64) void gate_max_kernel(vlm_recurrence_args p, int
 
 template <typename T>
 int run(const vlm_recurrence_args& a, int nseg, int ntok, hipStream_t st) {
-  const int gated = a.gated;
+  const int gated = a.gated == 1, rowgate = a.gated == 2;
   const int C = a.Dv + (gated ? 1 : 0);
   const int P = (a.D + DR - 1) / DR;
   if (P * CT > 1024) return VLM_ERR_SHAPE;
   int TB = 16;
-  auto lds = [&](int tb) { return (size_t)tb * (2 * P * DR + CT + 4 + P * CT) * sizeof(float); };
+  auto lds = [&](int tb) { return (size_t)tb * ((rowgate ? 3 : 2) * P * DR + CT + 4 + P * CT) * sizeof(float); };
   while (TB > 4 && lds(TB) > 48 * 1024) TB >>= 1;
   if (lds(TB) > 64 * 1024) return VLM_ERR_SHAPE;
   dim3 grid(nseg, a.H, (C + CT - 1) / CT), block(P * CT);
@@ -199,9 +229,11 @@ int run(const vlm_recurrence_args& a, int nseg, int ntok, hipStream_t st) {
     // the per-token maxima first: the scan kernel overwrites the slot's running maximum
     hipLaunchKernelGGL(gate_max_kernel<T>, dim3(nseg * a.H), dim3(64), 0, st, a, nseg);
     VLM_CHECK_LAUNCH();
-    hipLaunchKernelGGL((linear_recurrence_kernel<T, true>), grid, block, lds(TB), st, a, P, TB);
+    hipLaunchKernelGGL((linear_recurrence_kernel<T, 1>), grid, block, lds(TB), st, a, P, TB);
+  } else if (rowgate) {
+    hipLaunchKernelGGL((linear_recurrence_kernel<T, 2>), grid, block, lds(TB), st, a, P, TB);
   } else {
-    hipLaunchKernelGGL((linear_recurrence_kernel<T, false>), grid, block, lds(TB), st, a, P, TB);
+    hipLaunchKernelGGL((linear_recurrence_kernel<T, 0>), grid, block, lds(TB), st, a, P, TB);
   }
   VLM_CHECK_LAUNCH();
   if (gated)
@@ -218,12 +250,13 @@ int run(const vlm_recurrence_args& a, int nseg, int ntok, hipStream_t st) {
 
 extern "C" int vlm_linear_recurrence(const vlm_recurrence_args* a, int nseg, int ntok, int dtype, void* stream) {
   if (!a || nseg < 0 || ntok < 0) return VLM_ERR_ARG;
-  if (!a->q || !a->k || !a->v || !a->g || !a->state || !a->raw || !a->out || !a->seg_start || !a->seg_slot || !a->seg_pos0)
+  if (a->gated < 0 || a->gated > 2 || a->gate_act < 0 || a->gate_act > 2 || (a->gated == 2 && a->rot_dims)) return VLM_ERR_ARG;
+  if (!a->q || !a->k || !a->v || (!a->g && a->gate_act != 2) || !a->state || !a->raw || !a->out || !a->seg_start || !a->seg_slot || !a->seg_pos0)
     return VLM_ERR_ARG;
   if (a->H <= 0 || a->D <= 0 || a->Dv <= 0 || a->rot_dims < 0 || a->rot_dims > a->D || (a->rot_dims & 1)) return VLM_ERR_ARG;
   if (a->rot_dims && !a->inv_freq) return VLM_ERR_ARG;
-  if (a->gated ? (!a->ipre || !a->fpre || !a->ib || !a->fb || !a->mstate || !a->mtok || !a->mprev || !(a->cap > 0.f)) : !a->decay) return VLM_ERR_ARG;
-  if (a->ldq < (long)a->H * a->D || a->ldk < (long)a->H * a->D || a->ldv < (long)a->H * a->Dv || a->ldg < (long)a->H * a->Dv ||
+  if (a->gated == 2 ? false : a->gated ? (!a->ipre || !a->fpre || !a->ib || !a->fb || !a->mstate || !a->mtok || !a->mprev || !(a->cap > 0.f)) : !a->decay) return VLM_ERR_ARG;
+  if (a->ldq < (long)a->H * a->D || a->ldk < (long)a->H * a->D || a->ldv < (long)a->H * a->Dv || (a->g && a->ldg < (long)a->H * a->Dv) ||
       a->ldo < (long)a->H * a->Dv)
     return VLM_ERR_ARG;
   if (nseg == 0 || ntok == 0) return VLM_OK;

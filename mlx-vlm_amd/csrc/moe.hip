@@ -10,6 +10,12 @@
 //                        second normalisation over the chosen ones; and group-limited: consecutive experts are cut into
 //                        `groups` blocks of one size, a block ranks by its best expert, and the choice is made among the
 //                        experts of the `keep` top-ranked blocks (lowest index wins a tie).  groups = keep = 1: no limit.
+//   vlm_moe_route_sigmoid  scores s = sigmoid(z) per expert; the choice is made on s + correction (a per-expert offset that enters
+//                        nothing but the choice), limited to the `keep` best blocks of experts, a block ranking by the SUM of its
+//                        `group_top` largest choice scores; the experts of the other blocks cannot be chosen whatever their
+//                        scores (not even when the kept ones are negative); weights = the chosen s, divided by their sum + 1e-20
+//                        (when normalise), times scale.  The sigmoid of `extra` further logit columns is handed out beside the
+//                        table: the gate of an expert that every token uses.
 //   vlm_glu_rows         out[t][c] = act(g[t][c]) * u[t][c]; act: 0 = tanh-form gelu, 1 = silu, 2 = sigmoid.  With a route table:
 //                        E stacked experts of ff output columns, out[t][e ff + j] = act(g[t][e estride + j]) * u[t][e estride + j]
 //                        * route[t][e] (estride: the distance of two experts' columns in g and u, e.g. 2 ff when every expert's
@@ -123,6 +129,106 @@ __global__ __launch_bounds__(256) void moe_route_kernel(const float* __restrict_
   }
 }
 
+// one wave per token; lane l owns experts l, l + 64, ... (bit i of `taken`: the lane's i-th expert is chosen or not eligible)
+__global__ __launch_bounds__(256) void moe_route_sigmoid_kernel(const float* __restrict__ z, long ldz, int T, int E, int top, int groups,
+                                                                int keep, int group_top, const float* __restrict__ corr, int normalise,
+                                                                float scale, int extra, float* __restrict__ extra_out,
+                                                                float* __restrict__ gate, int* __restrict__ idx, float* __restrict__ wgt) {
+  const int t = blockIdx.x * 4 + (threadIdx.x >> 6), lane = threadIdx.x & 63;
+  if (t >= T) return;
+  const float* zr = z + (long)t * ldz;
+  for (int e = lane; e < E; e += 64) gate[(long)t * E + e] = 0.f;
+  for (int e = lane; e < extra; e += 64) extra_out[(long)t * extra + e] = 1.f / (1.f + expf(-zr[E + e]));
+  auto choice = [&](int e) { return 1.f / (1.f + expf(-zr[e])) + (corr ? corr[e] : 0.f); };
+  unsigned taken = 0u;
+  if (groups > 1 && keep < groups) {
+    const int gsz = E / groups;
+    // lane g (groups <= 64): the sum of the group_top largest choice scores of block g, members taken in index order
+    float gscore = -INFINITY;
+    if (lane < groups) {
+      float sum = 0.f;
+      int last = -1;
+      float lastv = INFINITY;
+      for (int k = 0; k < group_top && k < gsz; ++k) {   // k-th largest: the largest value below (lastv, last) in (value desc, index asc) order
+        float best = -INFINITY;
+        int bi = -1;
+        for (int j = 0; j < gsz; ++j) {
+          const float v = choice(lane * gsz + j);
+          const bool below = v < lastv || (v == lastv && j > last);
+          if (below && (bi < 0 || v > best)) {
+            best = v;
+            bi = j;
+          }
+        }
+        if (bi < 0) break;
+        sum += best;
+        lastv = best;
+        last = bi;
+      }
+      gscore = sum;
+    }
+    unsigned long long kept = 0ull;
+    for (int k = 0; k < keep; ++k) {
+      float best = (lane < groups && !((kept >> lane) & 1ull)) ? gscore : -INFINITY;
+      int bg = (lane < groups && !((kept >> lane) & 1ull)) ? lane : 0x7fffffff;
+#pragma unroll
+      for (int o = 32; o > 0; o >>= 1) {
+        const float ob = __shfl_xor(best, o);
+        const int og = __shfl_xor(bg, o);
+        if (og != 0x7fffffff && (bg == 0x7fffffff || ob > best || (ob == best && og < bg))) {
+          best = ob;
+          bg = og;
+        }
+      }
+      if (bg == 0x7fffffff) break;
+      kept |= 1ull << bg;
+    }
+    for (int e = lane, i = 0; e < E; e += 64, ++i)
+      if (!((kept >> (e / gsz)) & 1ull)) taken |= 1u << i;
+  }
+  float my_s = 0.f, denom = 0.f;
+  int my_idx = -1;
+  for (int j = 0; j < top; ++j) {
+    float best = -INFINITY;
+    int bi = 0x7fffffff;
+    for (int e = lane, i = 0; e < E; e += 64, ++i) {
+      if ((taken >> i) & 1u) continue;
+      const float v = choice(e);
+      if (bi == 0x7fffffff || v > best || (v == best && e < bi)) {
+        best = v;
+        bi = e;
+      }
+    }
+#pragma unroll
+    for (int o = 32; o > 0; o >>= 1) {
+      const float ob = __shfl_xor(best, o);
+      const int oi = __shfl_xor(bi, o);
+      if (oi != 0x7fffffff && (bi == 0x7fffffff || ob > best || (ob == best && oi < bi))) {
+        best = ob;
+        bi = oi;
+      }
+    }
+    if (bi == 0x7fffffff) break;
+    if (lane == (bi & 63)) taken |= 1u << (bi >> 6);
+    const float sj = 1.f / (1.f + expf(-zr[bi]));        // the weight uses the score WITHOUT the correction
+    if (lane == j) {
+      my_s = sj;
+      my_idx = bi;
+    }
+    denom += sj;                                         // chosen order, the same in every lane
+  }
+  const float w = my_idx < 0 ? 0.f : (normalise ? my_s / (denom + 1e-20f) : my_s) * scale;
+  if (lane < top) {
+    idx[(long)t * top + lane] = my_idx < 0 ? 0 : my_idx;
+    wgt[(long)t * top + lane] = w;
+  }
+  for (int j = 0; j < top; ++j) {
+    const int ej = __shfl(my_idx, j);
+    const float wj = __shfl(w, j);
+    if (ej >= 0 && lane == (ej & 63)) gate[(long)t * E + ej] = wj;
+  }
+}
+
 template <typename T>
 __global__ __launch_bounds__(256) void moe_relu2_gate_kernel(const T* __restrict__ up, long ldu, const float* __restrict__ gate, int E,
                                                              int ff, int shared, T* __restrict__ out, long ldo, int rows) {
@@ -185,6 +291,21 @@ extern "C" int vlm_moe_route_scored(const void* logits, int T, int E, int top, i
   if (T == 0) return VLM_OK;
   hipLaunchKernelGGL(moe_route_kernel, dim3((T + 3) / 4), dim3(256), 0, (hipStream_t)stream, (const float*)logits, T, E, top, 1, groups,
                      keep, scale, (float*)gate, (int*)idx, (float*)wgt);
+  VLM_CHECK_LAUNCH();
+  return VLM_OK;
+}
+
+extern "C" int vlm_moe_route_sigmoid(const void* logits, long ldz, int T, int E, int top, int groups, int keep, int group_top,
+                                     const void* correction, int normalise, float scale, int extra, void* extra_out, void* gate, void* idx,
+                                     void* wgt, void* stream) {
+  if (!logits || !gate || !idx || !wgt || T < 0 || E <= 0 || top <= 0 || top > E || groups <= 0 || keep <= 0 || keep > groups || E % groups ||
+      top > (long)keep * (E / groups) || group_top < 1 || extra < 0 || (extra && !extra_out) || ldz < (long)E + extra)
+    return VLM_ERR_ARG;
+  if (top > 64 || E > 2048 || groups > 64) return VLM_ERR_SHAPE;
+  if (T == 0) return VLM_OK;
+  hipLaunchKernelGGL(moe_route_sigmoid_kernel, dim3((T + 3) / 4), dim3(256), 0, (hipStream_t)stream, (const float*)logits, ldz, T, E, top,
+                     groups, keep, group_top, (const float*)correction, normalise, scale, extra, (float*)extra_out, (float*)gate, (int*)idx,
+                     (float*)wgt);
   VLM_CHECK_LAUNCH();
   return VLM_OK;
 }

@@ -1,6 +1,6 @@
 // Shared by the matrix-state recurrences (linear_recurrence.hip, delta_rule.hip): typed loads / stores and the finish pass
 // that turns the raw read-out o [token][head][Dv (+ 1)] (fp32) into the mixer's output row:
-//     o / denominator (gated form only)  ->  per-head unit RMS (eps)  ->  * normw[h][c] (optional)  ->  * silu or sigmoid of g
+//     o / denominator (gated form only)  ->  per-head unit RMS (eps)  ->  * normw[h][c] (optional)  ->  * silu or sigmoid of g (optional)
 #pragma once
 #include "common.hpp"
 
@@ -14,7 +14,7 @@ template <> __device__ __forceinline__ void st_f<float>(float* p, float v) { *p 
 template <> __device__ __forceinline__ void st_f<bf16_t>(bf16_t* p, float v) { *p = f2bf(v); }
 
 // grid (tokens, heads), one wave.  NORMALISER: column Dv of raw holds n . q, mtok the running maximum (exponential gating);
-// gate_act: 0 = silu(g), 1 = sigmoid(g)
+// gate_act: 0 = silu(g), 1 = sigmoid(g), 2 = no gate (g is not read)
 template <typename T, bool NORMALISER>
 __global__ __launch_bounds__(64) void recurrence_finish_kernel(const float* __restrict__ raw, int H, int Dv,
                                                                const float* __restrict__ mtok, float eps, const T* __restrict__ g,
@@ -39,6 +39,10 @@ __global__ __launch_bounds__(64) void recurrence_finish_kernel(const float* __re
   for (int c = lane; c < Dv; c += 64) {
     float x = o[c] * inv * r;
     if (normw) x *= ld_f(normw + (long)h * Dv + c);
+    if (gate_act == 2) {
+      st_f(op + c, x);
+      continue;
+    }
     const float gv = ld_f(gp + c), sg = 1.f / (1.f + expf(-gv));
     st_f(op + c, x * (gate_act == 0 ? gv * sg : sg));
   }

@@ -16,7 +16,7 @@
 //                              x[t] += rms(y * sigmoid(gate[t] + gate_bias)) * w      and h[t] = T(x[t]) for the next reader
 //   vlm_relu2_rows           out[t][j] = max(in[t][j], 0)^2
 //   vlm_scaled_add_rms       the residual step of a pre-norm sublayer and the norm of the next reader in one pass:
-//                              x[t] += mult * y[t]                                    (y may be NULL: norm only)
+//                              x[t] += mult * y[t] (+ mult2 * y2[t])                  (y may be NULL: norm only)
 //                              h[t] = x[t] * rsqrt(mean(x[t]^2) + eps) * (w_offset + w)   (w may be NULL: add only; w_offset 1
 //                                                                                      for weights kept as offsets from one)
 #include "common.hpp"
@@ -165,9 +165,10 @@ __global__ __launch_bounds__(256) void gated_rms_add_kernel(float* __restrict__ 
   }
 }
 
-template <typename T>
+template <typename T, typename HT>
 __global__ __launch_bounds__(256) void scaled_add_rms_kernel(float* __restrict__ x, const T* __restrict__ y, long ldy, float mult,
-                                                             const T* __restrict__ w, float w_offset, T* __restrict__ h, long ldh,
+                                                             const T* __restrict__ y2, long ldy2, float mult2,
+                                                             const T* __restrict__ w, float w_offset, HT* __restrict__ h, long ldh,
                                                              int D, float eps) {
   __shared__ float red[4];
   const long t = blockIdx.x;
@@ -177,6 +178,7 @@ __global__ __launch_bounds__(256) void scaled_add_rms_kernel(float* __restrict__
     float v = xr[d];
     if (y) {
       v = fmaf(mult, ld_f(y + t * ldy + d), v);
+      if (y2) v = fmaf(mult2, ld_f(y2 + t * ldy2 + d), v);
       xr[d] = v;
     }
     q += v * v;
@@ -309,13 +311,14 @@ extern "C" int vlm_relu2_rows(const void* in, long ldi, void* out, long ldo, int
   return VLM_OK;
 }
 
-extern "C" int vlm_scaled_add_rms(void* x, const void* y, long ldy, float mult, const void* w, float w_offset, void* h, long ldh, int rows,
-                                  int D, float eps, int dtype, void* stream) {
-  if (!x || !STREAM_ARGS_OK(rows, D) || (y && ldy < D) || (!y && !w) || (w && (!h || ldh < D))) return VLM_ERR_ARG;
+extern "C" int vlm_scaled_add_rms(void* x, const void* y, long ldy, float mult, const void* y2, long ldy2, float mult2, const void* w,
+                                  float w_offset, void* h, long ldh, int h_f32, int rows, int D, float eps, int dtype, void* stream) {
+  if (!x || !STREAM_ARGS_OK(rows, D) || (y && ldy < D) || (y2 && (!y || ldy2 < D)) || (!y && !w) || (w && (!h || ldh < D))) return VLM_ERR_ARG;
   if (rows == 0) return VLM_OK;
   hipStream_t st = (hipStream_t)stream;
-  if (dtype) hipLaunchKernelGGL(scaled_add_rms_kernel<float>, dim3(rows), dim3(256), 0, st, (float*)x, (const float*)y, ldy, mult, (const float*)w, w_offset, (float*)h, ldh, D, eps);
-  else hipLaunchKernelGGL(scaled_add_rms_kernel<bf16_t>, dim3(rows), dim3(256), 0, st, (float*)x, (const bf16_t*)y, ldy, mult, (const bf16_t*)w, w_offset, (bf16_t*)h, ldh, D, eps);
+  if (dtype) hipLaunchKernelGGL((scaled_add_rms_kernel<float, float>), dim3(rows), dim3(256), 0, st, (float*)x, (const float*)y, ldy, mult, (const float*)y2, ldy2, mult2, (const float*)w, w_offset, (float*)h, ldh, D, eps);
+  else if (h_f32) hipLaunchKernelGGL((scaled_add_rms_kernel<bf16_t, float>), dim3(rows), dim3(256), 0, st, (float*)x, (const bf16_t*)y, ldy, mult, (const bf16_t*)y2, ldy2, mult2, (const bf16_t*)w, w_offset, (float*)h, ldh, D, eps);
+  else hipLaunchKernelGGL((scaled_add_rms_kernel<bf16_t, bf16_t>), dim3(rows), dim3(256), 0, st, (float*)x, (const bf16_t*)y, ldy, mult, (const bf16_t*)y2, ldy2, mult2, (const bf16_t*)w, w_offset, (bf16_t*)h, ldh, D, eps);
   VLM_CHECK_LAUNCH();
   return VLM_OK;
 }

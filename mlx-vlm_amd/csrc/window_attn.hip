@@ -5,6 +5,7 @@
 //     s_ij = (q_i . k_j) * scale * temp[h]        j visible from i  <=>  0 <= i - j < window  (window <= 0: every j <= i)
 //     s_ij <- cap * tanh(s_ij / cap)              when a score cap is given (cap > 0)
 //     o_i  = sum_j softmax_j(s_ij) v_j * sigmoid(gate_i)        gate_i: one number per value column, or one per head
+//     sink: the softmax's denominator has one more term exp(0) that carries no value: p_ij = exp(s_ij) / (1 + sum_j exp(s_ij))
 //
 //   vlm_headnorm_rope_rows   x rows [T][heads][D] (T-typed) -> RMS norm per head (weight [D] shared by the heads, may be NULL)
 //                            -> rotation of the pairs (2 i, 2 i + 1), i < rot_dims / 2, by pos * inv_freq[i] -> fp32, either
@@ -42,7 +43,7 @@ __global__ __launch_bounds__(64) void headnorm_rope_kernel(const T* __restrict__
                                                            const int* __restrict__ tok_pos, const int* __restrict__ tok_seq,
                                                            const int* __restrict__ block_table, int max_pages,
                                                            float* __restrict__ out, const T* __restrict__ raw, long ldraw, int Draw,
-                                                           const T* __restrict__ raw_bias, T* __restrict__ raw_pool) {
+                                                           const T* __restrict__ raw_bias, T* __restrict__ raw_pool, int rot_half) {
   const long t = blockIdx.x;
   const int h = blockIdx.y, nh = gridDim.y, lane = threadIdx.x;
   const T* src = x + t * ldx + (long)h * D;
@@ -61,6 +62,34 @@ __global__ __launch_bounds__(64) void headnorm_rope_kernel(const T* __restrict__
   float r = norm ? 1.0f / sqrtf(ss / (float)D + eps) : 1.f;
   // (the multiplier is applied to the normed value as one more factor, so a design without it keeps its bits)
   const float mult = temp_every > 0 ? 1.f + temp_coef * logf((float)((pos + 1) / temp_every) + 1.f) : 1.f;
+  if (rot_half) {
+    // pairs (i, i + rot_dims / 2), turned FIRST and normed after: every lane evaluates its own dimension from the two inputs of
+    // its pair (the first half holds u, the second v: u' = u cos - v sin, v' = v cos + u sin), once for the sum of squares and
+    // once more for the store
+    const int half = rot_dims / 2;
+    auto turned = [&](int i) {
+      const float xi = ld_f(src + i) + (bs ? ld_f(bs + i) : 0.f);
+      if (i >= rot_dims) return xi;
+      const int j = i < half ? i + half : i - half;
+      const float xj = ld_f(src + j) + (bs ? ld_f(bs + j) : 0.f);
+      float sn, cs;
+      sincosf((float)pos * inv_freq[i < half ? i : j], &sn, &cs);
+      return i < half ? xi * cs - xj * sn : xi * cs + xj * sn;
+    };
+    float s2 = 0.f;
+    for (int i = lane; i < D; i += 64) {
+      const float v = turned(i);
+      s2 += v * v;
+    }
+#pragma unroll
+    for (int o = 32; o > 0; o >>= 1) s2 += __shfl_xor(s2, o);
+    r = norm ? 1.0f / sqrtf(s2 / (float)D + eps) : 1.f;
+    for (int i = lane; i < D; i += 64) {
+      float v = turned(i) * r * (w ? ld_f(w + i) : 1.f);
+      if (temp_every > 0) v *= mult;
+      dst[i] = v;
+    }
+  } else
   for (int i = lane; i < D / 2 + (D & 1); i += 64) {     // one pair per lane and trip (an odd last dimension passes alone)
     const int i0 = 2 * i, i1 = 2 * i + 1;
     float u = (ld_f(src + i0) + (bs ? ld_f(bs + i0) : 0.f)) * r * (w ? ld_f(w + i0) : 1.f);
@@ -97,7 +126,7 @@ __global__ __launch_bounds__(256) void window_attn_block_kernel(const float* __r
                                                                 const int* __restrict__ qb_count, const int* __restrict__ tok_seq,
                                                                 const int* __restrict__ tok_pos, const int* __restrict__ block_table,
                                                                 int max_pages, int H, int KH, int D, int Dv, float scale,
-                                                                const T* __restrict__ temp, int window, float cap, const T* __restrict__ gate,
+                                                                const T* __restrict__ temp, int window, float cap, int sink, const T* __restrict__ gate,
                                                                 long ldgate, int gate_head, T* __restrict__ out, long ldo) {
   extern __shared__ __align__(16) float smem[];
   const int DP = (D + 3) & ~3, KP = DP + 4, VP = NACC * 16;
@@ -192,7 +221,7 @@ __global__ __launch_bounds__(256) void window_attn_block_kernel(const float* __r
   __syncthreads();
   if (r16 < nq) {
     const long t = t0 + r16;
-    const float inv = 1.f / lrun[r16];
+    const float inv = 1.f / (lrun[r16] + (sink ? expf(-mrun[r16]) : 0.f));
 #pragma unroll
     for (int b = 0; b < NACC; ++b) {
       const int c = l16 + 16 * b;
@@ -211,7 +240,7 @@ __global__ __launch_bounds__(256) void window_attn_row_kernel(const float* __res
                                                               const T* __restrict__ vpool, const int* __restrict__ tok_seq,
                                                               const int* __restrict__ tok_pos, const int* __restrict__ block_table,
                                                               int max_pages, int H, int KH, int D, int Dv, float scale,
-                                                              const T* __restrict__ temp, int window, float cap, const T* __restrict__ gate,
+                                                              const T* __restrict__ temp, int window, float cap, int sink, const T* __restrict__ gate,
                                                               long ldgate, int gate_head, T* __restrict__ out, long ldo) {
   extern __shared__ __align__(16) float smem[];
   float* qs = smem;              // [D]
@@ -270,7 +299,7 @@ __global__ __launch_bounds__(256) void window_attn_row_kernel(const float* __res
     }
     __syncthreads();
   }
-  const float inv = 1.f / l_run;
+  const float inv = 1.f / (l_run + (sink ? expf(-m_run) : 0.f));
 #pragma unroll
   for (int a = 0; a < NACC; ++a) {
     const int c = tid + a * 256;
@@ -304,7 +333,7 @@ __global__ __launch_bounds__(256) void window_attn_row_vec_kernel(const float* _
                                                                   const T* __restrict__ vpool, const int* __restrict__ tok_seq,
                                                                   const int* __restrict__ tok_pos, const int* __restrict__ block_table,
                                                                   int max_pages, int H, int KH, int D, int Dv, float scale,
-                                                                  const T* __restrict__ temp, int window, float cap, const T* __restrict__ gate,
+                                                                  const T* __restrict__ temp, int window, float cap, int sink, const T* __restrict__ gate,
                                                                   long ldgate, int gate_head, T* __restrict__ out, long ldo) {
   extern __shared__ __align__(16) float smem[];
   float* qs = smem;                  // [D]
@@ -387,7 +416,7 @@ __global__ __launch_bounds__(256) void window_attn_row_vec_kernel(const float* _
 #pragma unroll
   for (int i = 0; i < 8; ++i) part[tid * 8 + i] = acc[i];
   __syncthreads();
-  const float inv = 1.f / l_run;
+  const float inv = 1.f / (l_run + (sink ? expf(-m_run) : 0.f));
   for (int c = tid; c < Dv; c += 256) {
     float o = 0.f;
     for (int pp = 0; pp < nparts; ++pp) o += part[(pp * ngroups + c / 8) * 8 + (c & 7)];
@@ -411,12 +440,12 @@ static int headnorm_launch(const vlm_headnorm_args* a, int rows, int dtype, void
     hipLaunchKernelGGL(headnorm_rope_kernel<float>, dim3(rows, a->heads), dim3(64), 0, st, (const float*)a->x, a->ldx, a->D,
                        (const float*)a->bias, (const float*)a->w, a->norm, a->eps, a->rot_dims, a->inv_freq, a->temp_coef, a->temp_every,
                        a->tok_pos, a->tok_seq, a->block_table, a->max_pages, a->out, (const float*)a->raw, a->ldraw, a->Draw,
-                       (const float*)a->raw_bias, (float*)a->raw_pool);
+                       (const float*)a->raw_bias, (float*)a->raw_pool, a->rot_half);
   else
     hipLaunchKernelGGL(headnorm_rope_kernel<bf16_t>, dim3(rows, a->heads), dim3(64), 0, st, (const bf16_t*)a->x, a->ldx, a->D,
                        (const bf16_t*)a->bias, (const bf16_t*)a->w, a->norm, a->eps, a->rot_dims, a->inv_freq, a->temp_coef, a->temp_every,
                        a->tok_pos, a->tok_seq, a->block_table, a->max_pages, a->out, (const bf16_t*)a->raw, a->ldraw, a->Draw,
-                       (const bf16_t*)a->raw_bias, (bf16_t*)a->raw_pool);
+                       (const bf16_t*)a->raw_bias, (bf16_t*)a->raw_pool, a->rot_half);
   VLM_CHECK_LAUNCH();
   return VLM_OK;
 }
@@ -442,7 +471,7 @@ extern "C" int vlm_headnorm_rope_rows(const void* x, long ldx, int heads, int D,
 
 extern "C" int vlm_window_attn_blocks(const void* q, const void* kpool, const void* vpool, const void* qb_start, const void* qb_count,
                                       int nblocks, const void* tok_seq, const void* tok_pos, const void* block_table, int max_pages,
-                                      int H, int KH, int D, int Dv, float scale, const void* temp, int window, float cap,
+                                      int H, int KH, int D, int Dv, float scale, const void* temp, int window, float cap, int sink,
                                       const void* gate, long ldgate, int gate_head, void* out, long ldo, int dtype, void* stream) {
   if (WINDOW_ARGS_BAD || !qb_start || !qb_count || nblocks < 0) return VLM_ERR_ARG;
   if (nblocks == 0) return VLM_OK;
@@ -455,7 +484,7 @@ extern "C" int vlm_window_attn_blocks(const void* q, const void* kpool, const vo
 #define GO(T, N)                                                                                                                    \
   hipLaunchKernelGGL((window_attn_block_kernel<T, N>), grid, dim3(256), lds, st, (const float*)q, (const float*)kpool, (const T*)vpool, \
                      (const int*)qb_start, (const int*)qb_count, (const int*)tok_seq, (const int*)tok_pos, (const int*)block_table,  \
-                     max_pages, H, KH, D, Dv, scale, (const T*)temp, window, cap, (const T*)gate, ldgate, gate_head, (T*)out, ldo)
+                     max_pages, H, KH, D, Dv, scale, (const T*)temp, window, cap, sink, (const T*)gate, ldgate, gate_head, (T*)out, ldo)
   if (dtype) {
     if (nacc == 4) GO(float, 4); else if (nacc == 8) GO(float, 8); else GO(float, 16);
   } else {
@@ -468,8 +497,8 @@ extern "C" int vlm_window_attn_blocks(const void* q, const void* kpool, const vo
 
 extern "C" int vlm_window_attn_rows(const void* q, const void* kpool, const void* vpool, const void* tok_seq, const void* tok_pos,
                                     const void* block_table, int max_pages, int H, int KH, int D, int Dv, float scale,
-                                    const void* temp, int window, float cap, const void* gate, long ldgate, int gate_head, void* out,
-                                    long ldo, int rows, int dtype, void* stream) {
+                                    const void* temp, int window, float cap, int sink, const void* gate, long ldgate, int gate_head,
+                                    void* out, long ldo, int rows, int dtype, void* stream) {
   if (WINDOW_ARGS_BAD || rows < 0) return VLM_ERR_ARG;
   if (rows == 0) return VLM_OK;
   if (Dv > 1024 || D > 8192 || H > 65535) return VLM_ERR_SHAPE;
@@ -480,11 +509,11 @@ extern "C" int vlm_window_attn_rows(const void* q, const void* kpool, const void
     if (dtype)
       hipLaunchKernelGGL(window_attn_row_vec_kernel<float>, grid, dim3(256), ldsv, st, (const float*)q, (const float*)kpool,
                          (const float*)vpool, (const int*)tok_seq, (const int*)tok_pos, (const int*)block_table, max_pages, H, KH, D, Dv,
-                         scale, (const float*)temp, window, cap, (const float*)gate, ldgate, gate_head, (float*)out, ldo);
+                         scale, (const float*)temp, window, cap, sink, (const float*)gate, ldgate, gate_head, (float*)out, ldo);
     else
       hipLaunchKernelGGL(window_attn_row_vec_kernel<bf16_t>, grid, dim3(256), ldsv, st, (const float*)q, (const float*)kpool,
                          (const bf16_t*)vpool, (const int*)tok_seq, (const int*)tok_pos, (const int*)block_table, max_pages, H, KH, D,
-                         Dv, scale, (const bf16_t*)temp, window, cap, (const bf16_t*)gate, ldgate, gate_head, (bf16_t*)out, ldo);
+                         Dv, scale, (const bf16_t*)temp, window, cap, sink, (const bf16_t*)gate, ldgate, gate_head, (bf16_t*)out, ldo);
     VLM_CHECK_LAUNCH();
     return VLM_OK;
   }
@@ -492,7 +521,7 @@ extern "C" int vlm_window_attn_rows(const void* q, const void* kpool, const void
 #define GO(T, N)                                                                                                                    \
   hipLaunchKernelGGL((window_attn_row_kernel<T, N>), grid, dim3(256), lds, st, (const float*)q, (const float*)kpool, (const T*)vpool, \
                      (const int*)tok_seq, (const int*)tok_pos, (const int*)block_table, max_pages, H, KH, D, Dv, scale,              \
-                     (const T*)temp, window, cap, (const T*)gate, ldgate, gate_head, (T*)out, ldo)
+                     (const T*)temp, window, cap, sink, (const T*)gate, ldgate, gate_head, (T*)out, ldo)
   const int nacc = (Dv + 255) / 256;
   if (dtype) {
     if (nacc == 1) GO(float, 1); else if (nacc == 2) GO(float, 2); else GO(float, 4);

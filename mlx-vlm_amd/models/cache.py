@@ -647,8 +647,8 @@ class HybridPool(KVPool):
         """row_layers: {key: row width, or (row width, dtype)} for layers that write cached rows per token (key: the layer
         index, or any sortable key when a layer keeps several row caches, e.g. (layer, "k") / (layer, "v"));
         state_layers: {layer: (heads, rows, cols, has_scalar)}: fp32 state [heads, rows, cols] (+ one fp32 scalar per head);
-        aux_layers: {layer: shape}: further fp32 state per sequence slot, [max_seqs, *shape] (e.g. the last inputs of a
-        short convolution)"""
+        aux_layers: {key: shape}: further fp32 state per sequence slot, [max_seqs, *shape] (e.g. the last inputs of a
+        short convolution); key: the layer index, or (layer, name) when a layer carries several"""
         self.n_layers = n_layers
         self.n_kv_heads = self.head_dim = 0                    # (no per-head K / V pages in this pool)
         self.n_pages = (max_tokens + PAGE - 1) // PAGE
@@ -661,7 +661,7 @@ class HybridPool(KVPool):
         for l, w in row_layers.items():
             w, dt = (w if isinstance(w, tuple) else (w, dtype))
             self.rows[int(l) if not isinstance(l, tuple) else l] = torch.zeros(self.n_pages, PAGE, int(w), dtype=dt, device=device)
-        self.aux = {int(l): torch.zeros(max_seqs, *[int(d) for d in shape], dtype=torch.float32, device=device)
+        self.aux = {(l if isinstance(l, tuple) else int(l)): torch.zeros(max_seqs, *[int(d) for d in shape], dtype=torch.float32, device=device)
                     for l, shape in (aux_layers or {}).items()}
         self.state = {int(l): torch.zeros(max_seqs, h, r, c, dtype=torch.float32, device=device)
                       for l, (h, r, c, _) in state_layers.items()}
@@ -752,11 +752,12 @@ class RecurrentCache:
     @property
     def state(self):
         pool, s = self._seq.pool, self._seq.seq
-        out = [pool.state[self._layer][s]]
+        out = [pool.state[self._layer][s]] if self._layer in pool.state else []
         if self._layer in pool.scalar:
             out.append(pool.scalar[self._layer][s])
-        if self._layer in pool.aux:
-            out.append(pool.aux[self._layer][s])
+        for k in sorted(pool.aux, key=str):
+            if k == self._layer or (isinstance(k, tuple) and k[0] == self._layer):
+                out.append(pool.aux[k][s])
         return out
 
     @property

@@ -727,19 +727,41 @@ def glu_rows(g, u, act, out=None, route=None, E=0, ff=0, estride=0):
     return out
 
 
-def scaled_add_rms_(x, y=None, mult=1.0, w=None, w_offset=0.0, eps=1e-6, h=None):
-    """x += mult * y on the fp32 stream (y None: no add); then, with w: h = rms(x) * (w_offset + w) in w's dtype -> h (None
-    without w).  One pass: the residual step of a sublayer and the norm of the next reader."""
-    _dev(x, y, w, h)
+def scaled_add_rms_(x, y=None, mult=1.0, w=None, w_offset=0.0, eps=1e-6, h=None, y2=None, mult2=1.0, h_dtype=None):
+    """x += mult * y (+ mult2 * y2) on the fp32 stream (y None: no add); then, with w: h = rms(x) * (w_offset + w) -> h (None
+    without w), in w's dtype, or in fp32 with h_dtype=torch.float32 (a reader that goes on in fp32).  One pass: the residual step
+    of a sublayer and the norm of the next reader."""
+    _dev(x, y, y2, w, h)
     if x.dtype != torch.float32 or not x.is_contiguous():
         raise _lib.VlmHipError("scaled_add_rms: contiguous fp32 stream expected")
     if w is not None and h is None:
-        h = torch.empty(x.shape, dtype=w.dtype, device=x.device)
+        h = torch.empty(x.shape, dtype=h_dtype or w.dtype, device=x.device)
     t = y if y is not None else w
-    check(_lib.lib().vlm_scaled_add_rms(_p(x), _p(y), y.stride(0) if y is not None else 0, float(mult), _p(w), float(w_offset), _p(h),
-                                        h.stride(0) if h is not None else 0, x.shape[0], x.shape[1], float(eps), _f32(t), _stream()),
-          "scaled_add_rms")
+    if y2 is not None and (y is None or y2.dtype != y.dtype):
+        raise _lib.VlmHipError("scaled_add_rms: the second addend comes with a first one of the same dtype")
+    check(_lib.lib().vlm_scaled_add_rms(_p(x), _p(y), y.stride(0) if y is not None else 0, float(mult), _p(y2),
+                                        y2.stride(0) if y2 is not None else 0, float(mult2), _p(w), float(w_offset), _p(h),
+                                        h.stride(0) if h is not None else 0, int(h is not None and h.dtype == torch.float32), x.shape[0],
+                                        x.shape[1], float(eps), _f32(t), _stream()), "scaled_add_rms")
     return h
+
+
+def moe_route_sigmoid(logits, E, top, groups=1, keep=1, group_top=2, correction=None, normalise=True, scale=1.0, extra=0):
+    """fp32 logits [T, >= E + extra] -> (gate table fp32 [T, E], chosen int32 [T, top], weights fp32 [T, top], sigmoid of the extra
+    columns fp32 [T, extra] or None).  Scores sigmoid(z); the choice on scores + correction inside the `keep` best of `groups`
+    blocks of neighbouring experts (a block ranks by the sum of its group_top best choice scores); weights from the scores alone."""
+    _dev(logits, correction)
+    if logits.dtype != torch.float32 or (correction is not None and correction.dtype != torch.float32):
+        raise _lib.VlmHipError("moe_route_sigmoid: fp32 logits and correction expected")
+    T = logits.shape[0]
+    gate = torch.empty(T, E, dtype=torch.float32, device=logits.device)
+    idx = torch.empty(T, top, dtype=torch.int32, device=logits.device)
+    wgt = torch.empty(T, top, dtype=torch.float32, device=logits.device)
+    ex = torch.empty(T, extra, dtype=torch.float32, device=logits.device) if extra else None
+    check(_lib.lib().vlm_moe_route_sigmoid(_p(logits), logits.stride(0), T, int(E), int(top), int(groups), int(keep), int(group_top),
+                                           _p(correction), int(bool(normalise)), float(scale), int(extra), _p(ex), _p(gate), _p(idx), _p(wgt),
+                                           _stream()), "moe_route_sigmoid")
+    return gate, idx, wgt, ex
 
 
 def moe_relu2_gate(up, gate, E, ff, shared, out):
@@ -822,16 +844,17 @@ def headnorm_rope_rows(x, heads, D, w, eps, rot_dims, inv_freq, tok_pos, out, to
 
 
 def headnorm_rows(x, heads, D, tok_pos, out, eps=0.0, norm=True, w=None, bias=None, rot_dims=0, inv_freq=None, temp=None, tok_seq=None,
-                  block_table=None, raw=None, raw_dim=0, raw_bias=None, raw_pool=None):
+                  block_table=None, raw=None, raw_dim=0, raw_bias=None, raw_pool=None, rot_half=False):
     """headnorm_rope_rows with a bias added first, a norm without a weight (norm=True, w=None), a position multiplier
     temp = (coef, every): 1 + coef * ln(floor((pos + 1) / every) + 1), and value rows `raw` (2-D view [T, heads * raw_dim],
-    + raw_bias) copied into `raw_pool` in the same launch"""
+    + raw_bias) copied into `raw_pool` in the same launch; rot_half: the rotated pairs are (i, i + rot_dims / 2) and the rotation comes
+    before the norm"""
     _dev(x, w, bias, inv_freq, tok_pos, out, tok_seq, block_table, raw, raw_bias, raw_pool)
     if out.dtype != torch.float32:
         raise _lib.VlmHipError("headnorm_rows: fp32 output expected")
     a = _lib.HeadnormArgs()
     a.x, a.ldx, a.heads, a.D, a.bias, a.w, a.norm, a.eps = _p(x), x.stride(0), int(heads), int(D), _p(bias), _p(w), int(bool(norm)), float(eps)
-    a.rot_dims, a.inv_freq = int(rot_dims), _p(inv_freq)
+    a.rot_dims, a.inv_freq, a.rot_half = int(rot_dims), _p(inv_freq), int(bool(rot_half))
     if temp is not None:
         a.temp_coef, a.temp_every = float(temp[0]), int(temp[1])
     a.tok_pos, a.tok_seq, a.block_table = _p(tok_pos), _p(tok_seq), _p(block_table)
@@ -846,24 +869,55 @@ def headnorm_rows(x, heads, D, tok_pos, out, eps=0.0, norm=True, w=None, bias=No
 
 
 def window_attn_blocks(q, kpool, vpool, qb_start, qb_count, tok_seq, tok_pos, block_table, H, KH, D, Dv, scale, out, temp=None, window=0,
-                       gate=None, cap=0.0, gate_head=False):
+                       gate=None, cap=0.0, gate_head=False, sink=False):
     """prompt form of the windowed attention: q fp32 [T, H * D]; out / gate: 2-D views [T, H * Dv] in vpool's dtype (gate_head:
-    gate [T, H], one number per head); cap > 0: scores pass cap * tanh(. / cap)"""
+    gate [T, H], one number per head); cap > 0: scores pass cap * tanh(. / cap); sink: one more term exp(0) in the softmax's denominator"""
     _dev(q, kpool, vpool, qb_start, qb_count, tok_seq, tok_pos, block_table, out, temp, gate)
     check(_lib.lib().vlm_window_attn_blocks(_p(q), _p(kpool), _p(vpool), _p(qb_start), _p(qb_count), qb_start.numel(), _p(tok_seq),
                                             _p(tok_pos), _p(block_table), block_table.shape[1], int(H), int(KH), int(D), int(Dv),
-                                            float(scale), _p(temp), int(window), float(cap), _p(gate),
+                                            float(scale), _p(temp), int(window), float(cap), int(bool(sink)), _p(gate),
                                             gate.stride(0) if gate is not None else 0, int(bool(gate_head)), _p(out), out.stride(0),
                                             _f32(vpool), _stream()), "window_attn_blocks")
     return out
 
 
 def window_attn_rows(q, kpool, vpool, tok_seq, tok_pos, block_table, H, KH, D, Dv, scale, out, temp=None, window=0, gate=None, cap=0.0,
-                     gate_head=False):
+                     gate_head=False, sink=False):
     """decode form of the windowed attention (one workgroup per token and head)"""
     _dev(q, kpool, vpool, tok_seq, tok_pos, block_table, out, temp, gate)
     check(_lib.lib().vlm_window_attn_rows(_p(q), _p(kpool), _p(vpool), _p(tok_seq), _p(tok_pos), _p(block_table), block_table.shape[1],
-                                          int(H), int(KH), int(D), int(Dv), float(scale), _p(temp), int(window), float(cap), _p(gate),
-                                          gate.stride(0) if gate is not None else 0, int(bool(gate_head)), _p(out), out.stride(0),
+                                          int(H), int(KH), int(D), int(Dv), float(scale), _p(temp), int(window), float(cap), int(bool(sink)),
+                                          _p(gate), gate.stride(0) if gate is not None else 0, int(bool(gate_head)), _p(out), out.stride(0),
                                           q.shape[0], _f32(vpool), _stream()), "window_attn_rows")
     return out
+
+
+# ---------------------------------------------------------------------------------------------------------------------
+# Short convolutions with carried inputs and the selective state-space scan.
+def short_conv_rows(x, w, carry, tok_seq, tok_pos, cu, slot, pos0, bias=None, act=False, residual=False, out=None, out_dtype=None):
+    """Causal convolution over time on every channel of the rows x [T, >= C] (fp32 or w's dtype; a 2-D view with a row pitch):
+    out = (x if residual) + bias + sum_j w[:, j] * x(t - taps + 1 + j), silu when act.  carry fp32 [slots, taps - 1, C] holds each
+    sequence's last inputs; it is read for the tokens before the step's first one and then moved to the end of the segments
+    (cu / slot / pos0: the step's segment tables)."""
+    _dev(x, w, carry, tok_seq, tok_pos, cu, slot, pos0, bias, out)
+    C_, taps = w.shape
+    if out is None:
+        out = torch.empty(x.shape[0], C_, dtype=out_dtype or w.dtype, device=x.device)
+    if taps > 1 and (carry is None or carry.dtype != torch.float32 or tuple(carry.shape[1:]) != (taps - 1, C_)):
+        raise _lib.VlmHipError("short_conv_rows: fp32 carry [slots, taps - 1, channels] expected")
+    a = _lib.ShortConvArgs()
+    a.in_, a.ldin, a.in_f32 = _p(x), x.stride(0), int(x.dtype == torch.float32)
+    a.w, a.bias, a.C, a.taps, a.act, a.residual = _p(w), _p(bias), int(C_), int(taps), int(bool(act)), int(bool(residual))
+    a.carry, a.tok_seq, a.tok_pos = _p(carry), _p(tok_seq), _p(tok_pos)
+    a.seg_start, a.seg_slot, a.seg_pos0 = _p(cu), _p(slot), _p(pos0)
+    a.out, a.ldo, a.out_f32 = _p(out), out.stride(0), int(out.dtype == torch.float32)
+    f32 = _f32(w)
+    if f32 and not (a.in_f32 and a.out_f32):
+        raise _lib.VlmHipError("short_conv_rows: fp32 weights come with fp32 rows")
+    check(_lib.lib().vlm_short_conv_rows(C.byref(a), x.shape[0], f32, _stream()), "short_conv_rows")
+    check(_lib.lib().vlm_short_conv_carry(C.byref(a), slot.numel(), f32, _stream()), "short_conv_carry")
+    return out
+
+
+def selective_scan(args: "_lib.SelectiveScanArgs", nseg: int, ntok: int, dtype_f32: bool):
+    check(_lib.lib().vlm_selective_scan(C.byref(args), int(nseg), int(ntok), int(bool(dtype_f32)), _stream()), "selective_scan")
