@@ -85,7 +85,7 @@ def windowed_attention_mixer(h, W, p, m, eps):
     q = rms(h @ W[p + "q"].T + W[p + "q.b"], eps) * W[p + "q.norm"]
     k = rms(h @ W[p + "k"].T + W[p + "k.b"], eps) * W[p + "k.norm"]
     v = h @ W[p + "v"].T + W[p + "v.b"]
-    o = softmax_attention(q.view(T, H, D), k.view(T, G, D), v.view(T, G, Dv), float(m["scale"]), window=int(m["mask"]["size"]))
+    o = softmax_attention(q.view(T, H, D), k.view(T, G, D), v.view(T, G, Dv), float(m["scale"]), window=int((m.get("mask") or {}).get("size") or 0))
     return (o.reshape(T, H * Dv) * torch.sigmoid(h @ W[p + "g"].T)) @ W[p + "o"].T
 
 
@@ -204,7 +204,8 @@ def layer_runs(cfg):
 def forward(cfg, W, tokens):
     """-> (logits [T, vocab], [stream after every layer run])   W: {name: float64 tensor}"""
     eps = float(cfg["norm"]["eps"])
-    x = W["embed"][torch.as_tensor(tokens, dtype=torch.long)] * float(cfg["embedding"]["scale"])
+    x = W["embed"][torch.as_tensor(tokens, dtype=torch.long)] * float((cfg.get("embedding") or {}).get("scale", 1.0))
+    canon = bool((cfg.get("canon") or {}).get("taps", 0))
     x0 = x.clone()
     streams = []
     for i, readd in layer_runs(cfg):
@@ -212,7 +213,8 @@ def forward(cfg, W, tokens):
         if readd:
             x = x + x0
         h = scalar_norm(x, W[p + "norm1"], eps)
-        h = h + causal_conv(h, W[p + "canon1"])
+        if canon:
+            h = h + causal_conv(h, W[p + "canon1"])
         if L["type"] == "parallel":
             x = x + parallel_mixer(h, W, p + "mix.", L["mixer"], eps)
         elif L["type"] == "hgrn2":
