@@ -107,7 +107,7 @@ def main():
                     help="336x336 images per vision-tower call of the ViT throughput line (16 = the workload of rounds 1-4 is reported "
                          "next to it; 68 images, where every GEMM fills its last round of 256 workgroups, measured +0.4 %: the tail of a "
                          "launch is not a whole round)")
-    ap.add_argument("--workload", default="qwen2vl-2b", choices=["qwen2vl-2b", "nanollava", "qwen2vl-7b-b32", "qwen2vl-2b-w4", "phi35v-w4-b16", "idefics2-b8", "garesun-compare", "luvapel-compare", "tilalorn-compare"])
+    ap.add_argument("--workload", default="qwen2vl-2b", choices=["qwen2vl-2b", "nanollava", "qwen2vl-7b-b32", "qwen2vl-2b-w4", "phi35v-w4-b16", "idefics2-b8", "garesun-compare", "luvapel-compare", "tilalorn-compare", "dimudra-compare"])
     ap.add_argument("--kv-bits", type=int, default=0, help="phi35v-w4-b16: 8 = uniform 8-bit KV cache (kv_bits of the reference)")
     ap.add_argument("--no-cpu-baseline", action="store_true")
     ap.add_argument("--no-cpu-hf", action="store_true", help="skip the HuggingFace torch-CPU second opinion of cpu_baseline")
@@ -166,6 +166,11 @@ def main():
         # likewise: the Tilalorn design next to Garesun (latent attention and mixtures of experts on the same ragged step)
         from benchlib.tilalorn import workload_tilalorn_compare
         print(json.dumps(workload_tilalorn_compare(args)), flush=True)
+        return
+    if args.workload == "dimudra-compare":
+        # likewise: the Dimudra design next to Garesun (recurrences, attention and mixtures of experts with a shared expert)
+        from benchlib.dimudra import workload_dimudra_compare
+        print(json.dumps(workload_dimudra_compare(args)), flush=True)
         return
     if args.workload != "qwen2vl-2b":
         rank, ws, local = parallel.init()

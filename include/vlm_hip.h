@@ -792,6 +792,9 @@ typedef struct vlm_selective_scan_args {
   long ldx, ldz;
   const float *dt_pre, *B, *Cm;         /* fp32 rows: [C] at lddt, [N] at ldbc each */
   long lddt, ldbc;
+  const float* dt_low;                  /* with dt_w: dt_pre = W_dt dt_low is evaluated inside - fp32 rows [R] at lddt, dt_pre unused */
+  const void* dt_w;                     /* T [C][R] or NULL */
+  int R;
   const void *dt_bias, *A_log, *D;      /* T [C], T [C][N], T [C] */
   const int *seg_start, *seg_slot, *seg_pos0;
   float* state;

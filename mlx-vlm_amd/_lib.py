@@ -145,7 +145,7 @@ class ShortConvArgs(C.Structure):
 class SelectiveScanArgs(C.Structure):
     """vlm_selective_scan_args (include/vlm_hip.h)"""
     _fields_ = [("x", c_void_p), ("z", c_void_p), ("ldx", C.c_long), ("ldz", C.c_long), ("dt_pre", c_void_p), ("B", c_void_p),
-                ("Cm", c_void_p), ("lddt", C.c_long), ("ldbc", C.c_long), ("dt_bias", c_void_p), ("A_log", c_void_p), ("D", c_void_p),
+                ("Cm", c_void_p), ("lddt", C.c_long), ("ldbc", C.c_long), ("dt_low", c_void_p), ("dt_w", c_void_p), ("R", c_int), ("dt_bias", c_void_p), ("A_log", c_void_p), ("D", c_void_p),
                 ("seg_start", c_void_p), ("seg_slot", c_void_p), ("seg_pos0", c_void_p), ("state", c_void_p), ("out", c_void_p),
                 ("ldo", C.c_long), ("C", c_int), ("N", c_int)]
 

@@ -4,7 +4,8 @@
 //     S[c][n] <- exp(dt_c A[c][n]) S[c][n] + (dt_c x_c) B_n
 //     y_c = sum_n S[c][n] C_n + D_c x_c              out_c = y_c * silu(z_c)
 //
-// x (after its short convolution and activation) and z are T-typed projection rows; dt_pre, B and C are fp32 rows (everything
+// x (after its short convolution and activation) and z are T-typed projection rows; dt_pre (or the low-rank rows dt_low it is
+// projected from by W_dt), B and C are fp32 rows (everything
 // that enters the recurrence after the projections is fp32: step sizes, decays, their exponentials, the state).  One kernel
 // serves a prompt, a portion and a decoded token: a segment is a run of consecutive tokens of one sequence; the state is read
 // from the sequence's slot (zero when the segment starts at position 0: a slot that is used again needs no clearing), advanced
@@ -12,28 +13,47 @@
 //
 // Work split: workgroup of 256 lanes = 256 / P channels x P lanes per channel; lane p of a channel holds the states
 // n = p, p + P, ... (NS of them) in registers, so one token costs a lane NS exponentials and 2 NS FMAs; the read-out is summed
-// over the P lanes of a channel by an xor tree inside the wave (P <= 64 divides the wave).  Tokens are staged 16 at a time
-// through LDS: softplus is evaluated once per (token, channel) on the way in, y is gated and written coalesced on the way out.
+// over the P lanes of a channel inside the wave (DPP quad swaps and row mirrors up to 16 lanes, lane exchanges above: no LDS
+// traffic, the same tree whatever the cut).  Tokens are staged 16 at a time through LDS - softplus once per (token, channel) on
+// the way in, optionally with the step-size projection itself (dt_pre = W_dt dt_low, a dot of dt_rank per (token, channel)
+// against the staged low-rank rows) - and the 16 token updates are unrolled: only the state's FMA chain is sequential, the
+// exponentials, products and sums of later tokens overlap it.  A block shorter than 16 tokens is padded with dt = x = B = C = 0
+// (exp(0) * S + 0 leaves the state as it is).  y is gated and written coalesced on the way out.
 #include "common.hpp"
 #include "../../include/vlm_hip.h"
 #include "recurrence_finish.hpp"
 
 namespace {
 
+constexpr int TB = 16;
+
 __device__ __forceinline__ float softplus_f(float v) { return v > 20.f ? v : log1pf(expf(v)); }
 
-template <typename T, int NS>
-__global__ __launch_bounds__(256) void selective_scan_kernel(vlm_selective_scan_args a, int P, int TB) {
+// sum over the P lanes of a channel (P a power of two, groups aligned to P): every lane of the group ends with the same bits
+template <int P>
+__device__ __forceinline__ float group_sum(float v) {
+  if (P >= 2) v += vlm_dpp<0xB1, 0xf>(0.f, v);      // quad_perm [1,0,3,2]
+  if (P >= 4) v += vlm_dpp<0x4E, 0xf>(0.f, v);      // quad_perm [2,3,0,1]
+  if (P >= 8) v += vlm_dpp<0x141, 0xf>(0.f, v);     // row_half_mirror
+  if (P >= 16) v += vlm_dpp<0x140, 0xf>(0.f, v);    // row_mirror
+  if (P >= 32) v += __shfl_xor(v, 16);
+  if (P >= 64) v += __shfl_xor(v, 32);
+  return v;
+}
+
+template <typename T, int P, int NS>
+__global__ __launch_bounds__(256) void selective_scan_kernel(vlm_selective_scan_args a) {
   extern __shared__ __align__(16) float smem[];
-  const int CH = 256 / P, NP = P * NS;
+  constexpr int CH = 256 / P, NP = P * NS;
   float* dts = smem;                    // [TB][CH]
   float* xs = dts + TB * CH;            // [TB][CH]
   float* ys = xs + TB * CH;             // [TB][CH]
   float* Bs = ys + TB * CH;             // [TB][NP]
   float* Cs = Bs + TB * NP;             // [TB][NP]
+  float* lows = Cs + TB * NP;           // [TB][R] (fused step-size projection)
   const int seg = blockIdx.x, tid = threadIdx.x;
   const int ch = tid / P, p = tid % P, c0 = blockIdx.y * CH, c = c0 + ch;
-  const int C = a.C, N = a.N;
+  const int C = a.C, N = a.N, R = a.R;
   const int t_begin = a.seg_start[seg], t_end = a.seg_start[seg + 1];
   const int slot = a.seg_slot[seg], pos0 = a.seg_pos0[seg];
   const bool live = c < C;
@@ -49,23 +69,38 @@ __global__ __launch_bounds__(256) void selective_scan_kernel(vlm_selective_scan_
   const float Dc = live ? ld_f((const T*)a.D + c) : 0.f;
   for (int t0 = t_begin; t0 < t_end; t0 += TB) {
     const int nb = min(TB, t_end - t0);
-    for (int i = tid; i < nb * CH; i += 256) {
+    if (a.dt_w) {
+      for (int i = tid; i < nb * R; i += 256) lows[i] = a.dt_low[(long)(t0 + i / R) * a.lddt + i % R];
+      __syncthreads();
+    }
+    for (int i = tid; i < TB * CH; i += 256) {
       const int t = i / CH, cc = c0 + i % CH;
       float dt = 0.f, xv = 0.f;
-      if (cc < C) {
-        dt = softplus_f(a.dt_pre[(long)(t0 + t) * a.lddt + cc] + ld_f((const T*)a.dt_bias + cc));
+      if (t < nb && cc < C) {
+        float pre;
+        if (a.dt_w) {
+          const T* wr = (const T*)a.dt_w + (long)cc * R;
+          const float* lr = lows + t * R;
+          pre = 0.f;
+          for (int r = 0; r < R; ++r) pre = fmaf(ld_f(wr + r), lr[r], pre);
+        } else {
+          pre = a.dt_pre[(long)(t0 + t) * a.lddt + cc];
+        }
+        dt = softplus_f(pre + ld_f((const T*)a.dt_bias + cc));
         xv = ld_f((const T*)a.x + (long)(t0 + t) * a.ldx + cc);
       }
       dts[i] = dt;
       xs[i] = xv;
     }
-    for (int i = tid; i < nb * NP; i += 256) {
+    for (int i = tid; i < TB * NP; i += 256) {
       const int t = i / NP, n = i % NP;
-      Bs[i] = n < N ? a.B[(long)(t0 + t) * a.ldbc + n] : 0.f;
-      Cs[i] = n < N ? a.Cm[(long)(t0 + t) * a.ldbc + n] : 0.f;
+      const bool on = t < nb && n < N;
+      Bs[i] = on ? a.B[(long)(t0 + t) * a.ldbc + n] : 0.f;
+      Cs[i] = on ? a.Cm[(long)(t0 + t) * a.ldbc + n] : 0.f;
     }
     __syncthreads();
-    for (int t = 0; t < nb; ++t) {
+#pragma unroll
+    for (int t = 0; t < TB; ++t) {
       const float dt = dts[t * CH + ch], xv = xs[t * CH + ch];
       const float dtx = dt * xv;
       float part = 0.f;
@@ -75,7 +110,7 @@ __global__ __launch_bounds__(256) void selective_scan_kernel(vlm_selective_scan_
         s[j] = fmaf(expf(dt * A[j]), s[j], dtx * Bs[t * NP + n]);
         part = fmaf(s[j], Cs[t * NP + n], part);
       }
-      for (int o = P >> 1; o > 0; o >>= 1) part += __shfl_xor(part, o);
+      part = group_sum<P>(part);
       if (p == 0) ys[t * CH + ch] = fmaf(Dc, xv, part);
     }
     __syncthreads();
@@ -95,34 +130,43 @@ __global__ __launch_bounds__(256) void selective_scan_kernel(vlm_selective_scan_
   }
 }
 
+template <typename T, int P, int NS>
+void launch(const vlm_selective_scan_args& a, int nseg, hipStream_t st) {
+  constexpr int CH = 256 / P;
+  const size_t lds = (size_t)TB * (3 * CH + 2 * P * NS + (a.dt_w ? a.R : 0)) * sizeof(float);
+  hipLaunchKernelGGL((selective_scan_kernel<T, P, NS>), dim3(nseg, (a.C + CH - 1) / CH), dim3(256), lds, st, a);
+}
+
+template <typename T>
+int run(const vlm_selective_scan_args& a, int nseg, hipStream_t st) {
+  const int NS = a.N <= 64 ? 1 : (a.N <= 128 ? 2 : 4);
+  int P = 1;
+  while (P * NS < a.N) P <<= 1;
+  const int CH = 256 / P;
+  if ((size_t)TB * (3 * CH + 2 * P * NS + (a.dt_w ? a.R : 0)) * sizeof(float) > 64 * 1024 || (a.C + CH - 1) / CH > 65535) return VLM_ERR_SHAPE;
+  if (NS == 2) launch<T, 64, 2>(a, nseg, st);
+  else if (NS == 4) launch<T, 64, 4>(a, nseg, st);
+  else if (P == 1) launch<T, 1, 1>(a, nseg, st);
+  else if (P == 2) launch<T, 2, 1>(a, nseg, st);
+  else if (P == 4) launch<T, 4, 1>(a, nseg, st);
+  else if (P == 8) launch<T, 8, 1>(a, nseg, st);
+  else if (P == 16) launch<T, 16, 1>(a, nseg, st);
+  else if (P == 32) launch<T, 32, 1>(a, nseg, st);
+  else launch<T, 64, 1>(a, nseg, st);
+  VLM_CHECK_LAUNCH();
+  return VLM_OK;
+}
+
 }  // namespace
 
 extern "C" int vlm_selective_scan(const vlm_selective_scan_args* a, int nseg, int ntok, int dtype, void* stream) {
   if (!a || nseg < 0 || ntok < 0) return VLM_ERR_ARG;
-  if (!a->x || !a->z || !a->dt_pre || !a->B || !a->Cm || !a->dt_bias || !a->A_log || !a->D || !a->seg_start || !a->seg_slot ||
-      !a->seg_pos0 || !a->state || !a->out)
+  if (!a->x || !a->z || !a->B || !a->Cm || !a->dt_bias || !a->A_log || !a->D || !a->seg_start || !a->seg_slot || !a->seg_pos0 ||
+      !a->state || !a->out)
     return VLM_ERR_ARG;
-  if (a->C <= 0 || a->N <= 0 || a->ldx < a->C || a->ldz < a->C || a->lddt < a->C || a->ldbc < a->N || a->ldo < a->C) return VLM_ERR_ARG;
+  if (a->dt_w ? (!a->dt_low || a->R <= 0 || a->lddt < a->R) : (!a->dt_pre || a->lddt < a->C)) return VLM_ERR_ARG;
+  if (a->C <= 0 || a->N <= 0 || a->ldx < a->C || a->ldz < a->C || a->ldbc < a->N || a->ldo < a->C) return VLM_ERR_ARG;
   if (nseg == 0 || ntok == 0) return VLM_OK;
   if (a->N > 256 || nseg > 65535 * 16) return VLM_ERR_SHAPE;
-  const int NS = a->N <= 64 ? 1 : (a->N <= 128 ? 2 : 4);
-  int P = 1;
-  while (P * NS < a->N) P <<= 1;
-  const int CH = 256 / P;
-  int TB = 16;
-  auto lds = [&](int tb) { return (size_t)tb * (3 * CH + 2 * P * NS) * sizeof(float); };
-  if (lds(TB) > 48 * 1024) TB = 8;
-  const unsigned nblk = (unsigned)((a->C + CH - 1) / CH);
-  if (nblk > 65535) return VLM_ERR_SHAPE;
-  dim3 grid(nseg, nblk);
-  hipStream_t st = (hipStream_t)stream;
-#define GO(T, K) hipLaunchKernelGGL((selective_scan_kernel<T, K>), grid, dim3(256), lds(TB), st, *a, P, TB)
-  if (dtype) {
-    if (NS == 1) GO(float, 1); else if (NS == 2) GO(float, 2); else GO(float, 4);
-  } else {
-    if (NS == 1) GO(bf16_t, 1); else if (NS == 2) GO(bf16_t, 2); else GO(bf16_t, 4);
-  }
-#undef GO
-  VLM_CHECK_LAUNCH();
-  return VLM_OK;
+  return dtype ? run<float>(*a, nseg, (hipStream_t)stream) : run<bf16_t>(*a, nseg, (hipStream_t)stream);
 }

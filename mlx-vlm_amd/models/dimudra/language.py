@@ -5,8 +5,8 @@ Pre-norm layers on an fp32 residual stream x; a norm's weight is ONE number g (k
     proj = h @ [mixer projections]^T                                     one GEMM (rows packed at load)
     parallel  : left  = biased q / k / v, RMS norm over the whole q (k) row with a weight, keys into the paged fp32 cache, values
                         into theirs, sliding-window softmax attention without positions, elementwise sigmoid gate, W_o
-                right = [x | z] -> short convolution + silu on x (inputs carried) -> [dt | B | C] in fp32 -> step sizes
-                        softplus(W_dt dt + b) -> selective scan over the sequence's fp32 state, times silu(z), W_o
+                right = [x | z] -> short convolution + silu on x (inputs carried) -> [dt | B | C] in fp32 -> selective scan over
+                        the sequence's fp32 state (step sizes softplus(W_dt dt + b) evaluated in its staging), times silu(z), W_o
                 x += left_scale * left + right_scale * right
     hgrn2     : matrix-state recurrence whose forget gate per state row (bounded below) also sets the write strength,
                 q = silu(.), per-head RMS norm with a weight shared by the heads, W_o
@@ -119,6 +119,8 @@ class LanguageModel(RaggedLanguageModel):
                     down.append(("shared", g(p + "mlp.shared.down", (Wd, sff))))
                 ns.wff, ns.foff = pack_rows(up, T, dev)
                 ns.down, ns.doff = pack_cols(down, T, dev)
+                if ns.down.shape[1] % 64:           # whole K tiles for the matrix-core kernel's staging: zero columns meet zero activations
+                    ns.down = torch.nn.functional.pad(ns.down, (0, 64 - ns.down.shape[1] % 64)).contiguous()
             self._L.append(ns)
         # caches, states and carried inputs: one set per RUN of a layer
         self._runs = cfg.runs()
@@ -191,17 +193,16 @@ class LanguageModel(RaggedLanguageModel):
                             act=True, out=xc)
         # what enters the recurrence after the projections stays fp32: step-size logits, B and C
         dbc = self._linear(xc, ns.wx, out_dtype=f32)
-        dt_pre = self._linear(dbc[:, :R], ns.wdt, out_dtype=f32)
         out = torch.empty(Tn, _al8(C_), dtype=T, device=dev)[:, :C_]
         a = _lib.SelectiveScanArgs()
         a.x, a.ldx, a.z, a.ldz = xc.data_ptr(), xc.stride(0), xz[:, C_:].data_ptr(), xz.stride(0)
-        a.dt_pre, a.lddt = dt_pre.data_ptr(), dt_pre.stride(0)
+        a.dt_low, a.dt_w, a.R, a.lddt = dbc.data_ptr(), ns.wdt.data_ptr(), R, dbc.stride(0)     # W_dt is applied inside the scan's staging
         a.B, a.Cm, a.ldbc = dbc[:, R:].data_ptr(), dbc[:, R + N:].data_ptr(), dbc.stride(0)
         a.dt_bias, a.A_log, a.D = ns.dt_b.data_ptr(), ns.A_log.data_ptr(), ns.Dskip.data_ptr()
         a.seg_start, a.seg_slot, a.seg_pos0 = pl.cu.data_ptr(), pl.slot.data_ptr(), pl.pos0.data_ptr()
         a.state, a.out, a.ldo, a.C, a.N = self.pool.state[r].data_ptr(), out.data_ptr(), out.stride(0), C_, N
         ops.selective_scan(a, pl.nseg, Tn, T == f32)
-        keep += [xc, dbc, dt_pre]
+        keep += [xc, dbc]
         return out
 
     def _hgrn2(self, ns, proj, pl, r, keep):

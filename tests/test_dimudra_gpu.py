@@ -154,7 +154,11 @@ def test_selective_scan_against_a_token_loop_in_portions_and_reused_slots(T, C, 
         want[t] = (S @ Cm[t, :N].double() + D.double() * xv) * O.silu(z[t, :C].double())
     state = torch.full((3, 1, C, N), float("nan")).cuda()
 
-    def run(lo, hi, slot):
+    R = 7
+    low, wdt = torch.randn(n, R + 3, generator=g), torch.randn(C, R, generator=g).to(T)
+    want_fused = None
+
+    def run(lo, hi, slot, fused=False):
         out = torch.empty(hi - lo, C, dtype=T, device="cuda")
         xs, zs, dp, bs, cs = (t[lo:hi].cuda() for t in (x, z, dt_pre, Bm, Cm))
         keep = [t.cuda() for t in (dt_b, A_log, D)]
@@ -162,7 +166,11 @@ def test_selective_scan_against_a_token_loop_in_portions_and_reused_slots(T, C, 
         a = _lib.SelectiveScanArgs()
         a.x, a.ldx, a.z, a.ldz = xs.data_ptr(), xs.stride(0), zs.data_ptr(), zs.stride(0)
         a.dt_pre, a.lddt, a.B, a.Cm, a.ldbc = dp.data_ptr(), dp.stride(0), bs.data_ptr(), cs.data_ptr(), bs.stride(0)
-        a.dt_bias, a.A_log, a.D = (k.data_ptr() for k in keep)
+        if fused:                                                       # the step-size projection inside the scan
+            lw, wd = low[lo:hi].cuda(), wdt.cuda()
+            keep += [lw, wd]
+            a.dt_pre, a.dt_low, a.dt_w, a.R, a.lddt = None, lw.data_ptr(), wd.data_ptr(), R, lw.stride(0)
+        a.dt_bias, a.A_log, a.D = (k.data_ptr() for k in keep[:3])
         a.seg_start, a.seg_slot, a.seg_pos0 = cu.data_ptr(), sl.data_ptr(), p0.data_ptr()
         a.state, a.out, a.ldo, a.C, a.N = state.data_ptr(), out.data_ptr(), out.stride(0), C, N
         ops.selective_scan(a, 1, hi - lo, T == torch.float32)
@@ -177,6 +185,11 @@ def test_selective_scan_against_a_token_loop_in_portions_and_reused_slots(T, C, 
     assert torch.equal(parts, whole)                                    # token-by-token arithmetic: the cut does not show
     assert torch.equal(run(0, n, 2), whole)                             # a used slot, from position 0
     assert (state[2, 0].cpu().double() - S).abs().max() < 2e-4 * S.abs().max().clamp_min(1.0)
+    pre = (low[:, :R].double() @ wdt.double().T).float()
+    dt_pre.copy_(pre)
+    given, fused = run(0, n, 1), run(0, n, 1, fused=True)
+    assert (fused.double() - given.double()).abs().max() < tol * scale
+    assert torch.equal(torch.cat([run(a, b, 0, fused=True) for a, b in zip(cuts, cuts[1:])]), fused)
 
 
 @pytest.mark.parametrize("E,top,groups,keep", [(8, 3, 4, 2), (6, 2, 3, 2), (12, 4, 1, 1), (5, 5, 5, 5), (9, 1, 3, 1), (130, 6, 10, 3), (6, 2, 6, 3)])
