@@ -42,15 +42,17 @@ __device__ __forceinline__ float group_sum(float v) {
 }
 
 template <typename T, int P, int NS>
-__global__ __launch_bounds__(256) void selective_scan_kernel(vlm_selective_scan_args a) {
+__global__ __launch_bounds__(256) void selective_scan_kernel(vlm_selective_scan_args a, int wdt_lds, int TS) {
   extern __shared__ __align__(16) float smem[];
   constexpr int CH = 256 / P, NP = P * NS;
-  float* dts = smem;                    // [TB][CH]
-  float* xs = dts + TB * CH;            // [TB][CH]
-  float* ys = xs + TB * CH;             // [TB][CH]
-  float* Bs = ys + TB * CH;             // [TB][NP]
-  float* Cs = Bs + TB * NP;             // [TB][NP]
-  float* lows = Cs + TB * NP;           // [TB][R] (fused step-size projection)
+  // TS tokens (a multiple of TB) are staged at a time: the loads of a stage are exposed latency, so a stage is as long as LDS allows
+  float* dts = smem;                    // [TS][CH]
+  float* xs = dts + TS * CH;            // [TS][CH]
+  float* ys = xs + TS * CH;             // [TS][CH]
+  float* Bs = ys + TS * CH;             // [TS][NP]
+  float* Cs = Bs + TS * NP;             // [TS][NP]
+  float* lows = Cs + TS * NP;           // [TS][R] (fused step-size projection)
+  float* wdt = lows + TS * a.R;         // [CH][R + 1]: the block's rows of W_dt (when wdt_lds)
   const int seg = blockIdx.x, tid = threadIdx.x;
   const int ch = tid / P, p = tid % P, c0 = blockIdx.y * CH, c = c0 + ch;
   const int C = a.C, N = a.N, R = a.R;
@@ -67,22 +69,29 @@ __global__ __launch_bounds__(256) void selective_scan_kernel(vlm_selective_scan_
     s[j] = (on && pos0 > 0) ? S[n] : 0.f;
   }
   const float Dc = live ? ld_f((const T*)a.D + c) : 0.f;
-  for (int t0 = t_begin; t0 < t_end; t0 += TB) {
-    const int nb = min(TB, t_end - t0);
+  if (a.dt_w && wdt_lds)
+    for (int i = tid; i < CH * R; i += 256) wdt[(i / R) * (R + 1) + i % R] = c0 + i / R < C ? ld_f((const T*)a.dt_w + (long)(c0 + i / R) * R + i % R) : 0.f;
+  for (int t0 = t_begin; t0 < t_end; t0 += TS) {
+    const int nb = min(TS, t_end - t0);
     if (a.dt_w) {
       for (int i = tid; i < nb * R; i += 256) lows[i] = a.dt_low[(long)(t0 + i / R) * a.lddt + i % R];
       __syncthreads();
     }
-    for (int i = tid; i < TB * CH; i += 256) {
+    for (int i = tid; i < TS * CH; i += 256) {
       const int t = i / CH, cc = c0 + i % CH;
       float dt = 0.f, xv = 0.f;
       if (t < nb && cc < C) {
         float pre;
         if (a.dt_w) {
-          const T* wr = (const T*)a.dt_w + (long)cc * R;
           const float* lr = lows + t * R;
           pre = 0.f;
-          for (int r = 0; r < R; ++r) pre = fmaf(ld_f(wr + r), lr[r], pre);
+          if (wdt_lds) {
+            const float* wl = wdt + (i % CH) * (R + 1);
+            for (int r = 0; r < R; ++r) pre = fmaf(wl[r], lr[r], pre);
+          } else {
+            const T* wr = (const T*)a.dt_w + (long)cc * R;
+            for (int r = 0; r < R; ++r) pre = fmaf(ld_f(wr + r), lr[r], pre);
+          }
         } else {
           pre = a.dt_pre[(long)(t0 + t) * a.lddt + cc];
         }
@@ -92,26 +101,42 @@ __global__ __launch_bounds__(256) void selective_scan_kernel(vlm_selective_scan_
       dts[i] = dt;
       xs[i] = xv;
     }
-    for (int i = tid; i < TB * NP; i += 256) {
+    for (int i = tid; i < TS * NP; i += 256) {
       const int t = i / NP, n = i % NP;
       const bool on = t < nb && n < N;
       Bs[i] = on ? a.B[(long)(t0 + t) * a.ldbc + n] : 0.f;
       Cs[i] = on ? a.Cm[(long)(t0 + t) * a.ldbc + n] : 0.f;
     }
     __syncthreads();
+    for (int tc = 0; tc < nb; tc += TB) {
+    // three passes over 16 staged tokens, so that only the FMA chain of the state is sequential: (1) decays and inputs of every
+    // token, independent of the state; (2) the chain; (3) the sums over the channel's lanes, independent of each other
+    float e[TB][NS], bx[TB][NS], part[TB];
 #pragma unroll
     for (int t = 0; t < TB; ++t) {
-      const float dt = dts[t * CH + ch], xv = xs[t * CH + ch];
-      const float dtx = dt * xv;
-      float part = 0.f;
+      const float dt = dts[(tc + t) * CH + ch], dtx = dt * xs[(tc + t) * CH + ch];
 #pragma unroll
       for (int j = 0; j < NS; ++j) {
-        const int n = p + P * j;
-        s[j] = fmaf(expf(dt * A[j]), s[j], dtx * Bs[t * NP + n]);
-        part = fmaf(s[j], Cs[t * NP + n], part);
+        e[t][j] = expf(dt * A[j]);
+        bx[t][j] = dtx * Bs[(tc + t) * NP + p + P * j];
       }
-      part = group_sum<P>(part);
-      if (p == 0) ys[t * CH + ch] = fmaf(Dc, xv, part);
+    }
+#pragma unroll
+    for (int t = 0; t < TB; ++t) {
+      float acc = 0.f;
+#pragma unroll
+      for (int j = 0; j < NS; ++j) {
+        s[j] = fmaf(e[t][j], s[j], bx[t][j]);
+        acc = fmaf(s[j], Cs[(tc + t) * NP + p + P * j], acc);
+      }
+      part[t] = acc;
+    }
+#pragma unroll
+    for (int t = 0; t < TB; ++t) part[t] = group_sum<P>(part[t]);
+    if (p == 0) {
+#pragma unroll
+      for (int t = 0; t < TB; ++t) ys[(tc + t) * CH + ch] = fmaf(Dc, xs[(tc + t) * CH + ch], part[t]);
+    }
     }
     __syncthreads();
     for (int i = tid; i < nb * CH; i += 256) {
@@ -131,28 +156,33 @@ __global__ __launch_bounds__(256) void selective_scan_kernel(vlm_selective_scan_
 }
 
 template <typename T, int P, int NS>
-void launch(const vlm_selective_scan_args& a, int nseg, hipStream_t st) {
+void launch(const vlm_selective_scan_args& a, int nseg, int maxlen, hipStream_t st) {
   constexpr int CH = 256 / P;
-  const size_t lds = (size_t)TB * (3 * CH + 2 * P * NS + (a.dt_w ? a.R : 0)) * sizeof(float);
-  hipLaunchKernelGGL((selective_scan_kernel<T, P, NS>), dim3(nseg, (a.C + CH - 1) / CH), dim3(256), lds, st, a);
+  const size_t per_tok = (size_t)(3 * CH + 2 * P * NS + (a.dt_w ? a.R : 0)) * sizeof(float);
+  const size_t wl = a.dt_w ? (size_t)CH * (a.R + 1) * sizeof(float) : 0;
+  const int wdt_lds = wl && TB * per_tok + wl <= 60 * 1024;          // (else the rows are read from memory in the staging loop)
+  const size_t fixed = wdt_lds ? wl : 0;
+  int TS = TB;
+  (void)maxlen;             // (longer stages measured slower: the staging loop's loads are not overlapped across its trips)
+  hipLaunchKernelGGL((selective_scan_kernel<T, P, NS>), dim3(nseg, (a.C + CH - 1) / CH), dim3(256), TS * per_tok + fixed, st, a, wdt_lds, TS);
 }
 
 template <typename T>
-int run(const vlm_selective_scan_args& a, int nseg, hipStream_t st) {
+int run(const vlm_selective_scan_args& a, int nseg, int maxlen, hipStream_t st) {
   const int NS = a.N <= 64 ? 1 : (a.N <= 128 ? 2 : 4);
   int P = 1;
   while (P * NS < a.N) P <<= 1;
   const int CH = 256 / P;
   if ((size_t)TB * (3 * CH + 2 * P * NS + (a.dt_w ? a.R : 0)) * sizeof(float) > 64 * 1024 || (a.C + CH - 1) / CH > 65535) return VLM_ERR_SHAPE;
-  if (NS == 2) launch<T, 64, 2>(a, nseg, st);
-  else if (NS == 4) launch<T, 64, 4>(a, nseg, st);
-  else if (P == 1) launch<T, 1, 1>(a, nseg, st);
-  else if (P == 2) launch<T, 2, 1>(a, nseg, st);
-  else if (P == 4) launch<T, 4, 1>(a, nseg, st);
-  else if (P == 8) launch<T, 8, 1>(a, nseg, st);
-  else if (P == 16) launch<T, 16, 1>(a, nseg, st);
-  else if (P == 32) launch<T, 32, 1>(a, nseg, st);
-  else launch<T, 64, 1>(a, nseg, st);
+  if (NS == 2) launch<T, 64, 2>(a, nseg, maxlen, st);
+  else if (NS == 4) launch<T, 64, 4>(a, nseg, maxlen, st);
+  else if (P == 1) launch<T, 1, 1>(a, nseg, maxlen, st);
+  else if (P == 2) launch<T, 2, 1>(a, nseg, maxlen, st);
+  else if (P == 4) launch<T, 4, 1>(a, nseg, maxlen, st);
+  else if (P == 8) launch<T, 8, 1>(a, nseg, maxlen, st);
+  else if (P == 16) launch<T, 16, 1>(a, nseg, maxlen, st);
+  else if (P == 32) launch<T, 32, 1>(a, nseg, maxlen, st);
+  else launch<T, 64, 1>(a, nseg, maxlen, st);
   VLM_CHECK_LAUNCH();
   return VLM_OK;
 }
@@ -168,5 +198,5 @@ extern "C" int vlm_selective_scan(const vlm_selective_scan_args* a, int nseg, in
   if (a->C <= 0 || a->N <= 0 || a->ldx < a->C || a->ldz < a->C || a->ldbc < a->N || a->ldo < a->C) return VLM_ERR_ARG;
   if (nseg == 0 || ntok == 0) return VLM_OK;
   if (a->N > 256 || nseg > 65535 * 16) return VLM_ERR_SHAPE;
-  return dtype ? run<float>(*a, nseg, (hipStream_t)stream) : run<bf16_t>(*a, nseg, (hipStream_t)stream);
+  return dtype ? run<float>(*a, nseg, ntok, (hipStream_t)stream) : run<bf16_t>(*a, nseg, ntok, (hipStream_t)stream);      // (ntok bounds a segment's length)
 }
