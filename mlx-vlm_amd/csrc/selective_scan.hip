@@ -42,10 +42,12 @@ __device__ __forceinline__ float group_sum(float v) {
 }
 
 template <typename T, int P, int NS>
-__global__ __launch_bounds__(256) void selective_scan_kernel(vlm_selective_scan_args a, int wdt_lds, int TS) {
+__global__ __launch_bounds__(256) void selective_scan_kernel(vlm_selective_scan_args a, int wdt_lds) {
   extern __shared__ __align__(16) float smem[];
   constexpr int CH = 256 / P, NP = P * NS;
-  // TS tokens (a multiple of TB) are staged at a time: the loads of a stage are exposed latency, so a stage is as long as LDS allows
+  // (a stage is one block of TB tokens: with compile-time offsets the LDS reads of the unrolled updates need no address arithmetic;
+  //  stages of 64 tokens with run-time offsets measured 1.5 x slower)
+  constexpr int TS = TB;
   float* dts = smem;                    // [TS][CH]
   float* xs = dts + TS * CH;            // [TS][CH]
   float* ys = xs + TS * CH;             // [TS][CH]
@@ -108,7 +110,8 @@ __global__ __launch_bounds__(256) void selective_scan_kernel(vlm_selective_scan_
       Cs[i] = on ? a.Cm[(long)(t0 + t) * a.ldbc + n] : 0.f;
     }
     __syncthreads();
-    for (int tc = 0; tc < nb; tc += TB) {
+    {
+    constexpr int tc = 0;
     // three passes over 16 staged tokens, so that only the FMA chain of the state is sequential: (1) decays and inputs of every
     // token, independent of the state; (2) the chain; (3) the sums over the channel's lanes, independent of each other
     float e[TB][NS], bx[TB][NS], part[TB];
@@ -162,9 +165,8 @@ void launch(const vlm_selective_scan_args& a, int nseg, int maxlen, hipStream_t 
   const size_t wl = a.dt_w ? (size_t)CH * (a.R + 1) * sizeof(float) : 0;
   const int wdt_lds = wl && TB * per_tok + wl <= 60 * 1024;          // (else the rows are read from memory in the staging loop)
   const size_t fixed = wdt_lds ? wl : 0;
-  int TS = TB;
-  (void)maxlen;             // (longer stages measured slower: the staging loop's loads are not overlapped across its trips)
-  hipLaunchKernelGGL((selective_scan_kernel<T, P, NS>), dim3(nseg, (a.C + CH - 1) / CH), dim3(256), TS * per_tok + fixed, st, a, wdt_lds, TS);
+  (void)maxlen;
+  hipLaunchKernelGGL((selective_scan_kernel<T, P, NS>), dim3(nseg, (a.C + CH - 1) / CH), dim3(256), TB * per_tok + fixed, st, a, wdt_lds);
 }
 
 template <typename T>
