@@ -89,9 +89,11 @@ __global__ __launch_bounds__(256) void selective_scan_kernel(vlm_selective_scan_
           pre = 0.f;
           if (wdt_lds) {
             const float* wl = wdt + (i % CH) * (R + 1);
-            for (int r = 0; r < R; ++r) pre = fmaf(wl[r], lr[r], pre);
+#pragma unroll 8
+            for (int r = 0; r < R; ++r) pre = fmaf(wl[r], lr[r], pre);      // (unrolled: eight pairs of LDS reads in flight per wait)
           } else {
             const T* wr = (const T*)a.dt_w + (long)cc * R;
+#pragma unroll 8
             for (int r = 0; r < R; ++r) pre = fmaf(ld_f(wr + r), lr[r], pre);
           }
         } else {
