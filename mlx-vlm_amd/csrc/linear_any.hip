@@ -76,6 +76,55 @@ __global__ __launch_bounds__(256) void linear_any_kernel(const TA* __restrict__ 
   }
 }
 
+// the same product on 16 x 64 output tiles (one row x four columns per lane) for shapes that give the 64 x 64 tiling too few
+// workgroups to fill the chip: few rows, or few output columns (router logits, low-rank maps).  Every output is the same FMA
+// chain over ascending k as in the 64 x 64 kernel - the same bits - so the choice between the two may depend on the row count.
+constexpr int SM = 16;
+template <typename TA, typename TW, typename TC>
+__global__ __launch_bounds__(256) void linear_any_rows16_kernel(const TA* __restrict__ A, const TW* __restrict__ W, TC* __restrict__ C,
+                                                                int M, int N, int K, long lda, long ldw, long ldc, long sA, long sW,
+                                                                long sC, int accumulate) {
+  __shared__ float As[BK][SM + 1];
+  __shared__ float Ws[BK][BN + 4];
+  const int b = blockIdx.z;
+  A += (long)b * sA;
+  W += (long)b * sW;
+  C += (long)b * sC;
+  const int m0 = blockIdx.y * SM, n0 = blockIdx.x * BN;
+  const int tid = threadIdx.x;
+  const int tm = tid / 16, tn = (tid % 16) * 4;
+  float acc[4] = {};
+  for (int k0 = 0; k0 < K; k0 += BK) {
+    {
+      const int r = tid >> 4, k = k0 + (tid & 15);           // 16 rows x 16 k of A: one element per lane
+      As[tid & 15][r] = (m0 + r < M && k < K) ? ld_f(A + (long)(m0 + r) * lda + k) : 0.f;
+    }
+    const int r = tid >> 2, kk = (tid & 3) * 4;             // 64 rows x 16 k of W: lane -> (row, 4 consecutive k)
+#pragma unroll
+    for (int j = 0; j < 4; ++j) {
+      const int k = k0 + kk + j;
+      Ws[kk + j][r] = (n0 + r < N && k < K) ? ld_f(W + (long)(n0 + r) * ldw + k) : 0.f;
+    }
+    __syncthreads();
+#pragma unroll
+    for (int k = 0; k < BK; ++k) {
+      const float a = As[k][tm];
+#pragma unroll
+      for (int j = 0; j < 4; ++j) acc[j] = fmaf(a, Ws[k][tn + j], acc[j]);
+    }
+    __syncthreads();
+  }
+  const int m = m0 + tm;
+  if (m >= M) return;
+#pragma unroll
+  for (int j = 0; j < 4; ++j) {
+    const int n = n0 + tn + j;
+    if (n >= N) continue;
+    TC* c = C + (long)m * ldc + n;
+    st_f(c, accumulate ? ld_f(c) + acc[j] : acc[j]);
+  }
+}
+
 // few rows (decode steps): the weights are the traffic, so W is read ONCE for all rows.  One wave per output column, lanes
 // across k (coalesced), up to 8 row accumulators per lane, xor-butterfly sum: a fixed order, so a row's result is still a
 // function of that row alone.  Sum order differs from the tile kernel's (rounding only); not used when everything is fp32.
@@ -177,6 +226,11 @@ int launch(const void* A, const void* W, void* C, int M, int N, int K, long lda,
   if (M <= 8 && !all_f32) {
     dim3 grid((N + 3) / 4, 1, batch);
     hipLaunchKernelGGL((linear_rows_kernel<TA, TW, TC>), grid, dim3(256), 0, st, (const TA*)A, (const TW*)W, (TC*)C, M, N, K, lda,
+                       ldw, ldc, sA, sW, sC, accumulate);
+  } else if ((long)((N + BN - 1) / BN) * ((M + BM - 1) / BM) * batch < 256) {
+    // fewer 64 x 64 tiles than compute units: 16-row tiles (the same bits per output)
+    dim3 grid((N + BN - 1) / BN, (M + SM - 1) / SM, batch);
+    hipLaunchKernelGGL((linear_any_rows16_kernel<TA, TW, TC>), grid, dim3(256), 0, st, (const TA*)A, (const TW*)W, (TC*)C, M, N, K, lda,
                        ldw, ldc, sA, sW, sC, accumulate);
   } else {
     dim3 grid((N + BN - 1) / BN, (M + BM - 1) / BM, batch);
