@@ -18,7 +18,8 @@
 // the way in, optionally with the step-size projection itself (dt_pre = W_dt dt_low, a dot of dt_rank per (token, channel)
 // against the staged low-rank rows) - and the 16 token updates are unrolled: only the state's FMA chain is sequential, the
 // exponentials, products and sums of later tokens overlap it.  A block shorter than 16 tokens is padded with dt = x = B = C = 0
-// (exp(0) * S + 0 leaves the state as it is).  y is gated and written coalesced on the way out.
+// (exp(0) * S + 0 leaves the state as it is).  The global loads of a stage are issued into registers one stage ahead, so they
+// are in flight while the stage before is computed.  y is gated and written coalesced on the way out.
 #include "common.hpp"
 #include "../../include/vlm_hip.h"
 #include "recurrence_finish.hpp"
@@ -41,26 +42,28 @@ __device__ __forceinline__ float group_sum(float v) {
   return v;
 }
 
+constexpr int LMAX = 16;      // low-rank rows of a stage held in registers: 16 x 256 values = 16 tokens of dt_rank <= 256
+
 template <typename T, int P, int NS>
 __global__ __launch_bounds__(256) void selective_scan_kernel(vlm_selective_scan_args a, int wdt_lds) {
   extern __shared__ __align__(16) float smem[];
   constexpr int CH = 256 / P, NP = P * NS;
-  // (a stage is one block of TB tokens: with compile-time offsets the LDS reads of the unrolled updates need no address arithmetic;
-  //  stages of 64 tokens with run-time offsets measured 1.5 x slower)
-  constexpr int TS = TB;
-  float* dts = smem;                    // [TS][CH]
-  float* xs = dts + TS * CH;            // [TS][CH]
-  float* ys = xs + TS * CH;             // [TS][CH]
-  float* Bs = ys + TS * CH;             // [TS][NP]
-  float* Cs = Bs + TS * NP;             // [TS][NP]
-  float* lows = Cs + TS * NP;           // [TS][R] (fused step-size projection)
-  float* wdt = lows + TS * a.R;         // [CH][R + 1]: the block's rows of W_dt (when wdt_lds)
+  constexpr int EX = (TB * CH + 255) / 256, EB = (TB * NP + 255) / 256;      // per-lane elements of a stage: channel rows, B / C rows
+  float* dts = smem;                    // [TB][CH]
+  float* xs = dts + TB * CH;            // [TB][CH]
+  float* zs = xs + TB * CH;             // [TB][CH]
+  float* ys = dts;                      // [TB][CH]: y takes the place of dt - a channel's lanes sit in ONE wave, which has read the
+                                        // channel's dt (first pass) before its lane 0 writes y (last pass)
+  float* Bs = zs + TB * CH;             // [TB][NP]
+  float* Cs = Bs + TB * NP;             // [TB][NP]
+  float* lows = Cs + TB * NP;           // [TB][R] (fused step-size projection)
+  float* wdt = lows + TB * a.R;         // [CH][R + 1]: the block's rows of W_dt (when wdt_lds)
   const int seg = blockIdx.x, tid = threadIdx.x;
   const int ch = tid / P, p = tid % P, c0 = blockIdx.y * CH, c = c0 + ch;
   const int C = a.C, N = a.N, R = a.R;
   const int t_begin = a.seg_start[seg], t_end = a.seg_start[seg + 1];
   const int slot = a.seg_slot[seg], pos0 = a.seg_pos0[seg];
-  const bool live = c < C;
+  const bool live = c < C, fused = a.dt_w != nullptr;
   float A[NS], s[NS];
   float* S = a.state + ((long)slot * C + (live ? c : 0)) * N;
 #pragma unroll
@@ -71,45 +74,98 @@ __global__ __launch_bounds__(256) void selective_scan_kernel(vlm_selective_scan_
     s[j] = (on && pos0 > 0) ? S[n] : 0.f;
   }
   const float Dc = live ? ld_f((const T*)a.D + c) : 0.f;
-  if (a.dt_w && wdt_lds)
+  if (fused && wdt_lds)
     for (int i = tid; i < CH * R; i += 256) wdt[(i / R) * (R + 1) + i % R] = c0 + i / R < C ? ld_f((const T*)a.dt_w + (long)(c0 + i / R) * R + i % R) : 0.f;
-  for (int t0 = t_begin; t0 < t_end; t0 += TS) {
-    const int nb = min(TS, t_end - t0);
-    if (a.dt_w) {
-      for (int i = tid; i < nb * R; i += 256) lows[i] = a.dt_low[(long)(t0 + i / R) * a.lddt + i % R];
-      __syncthreads();
+  float bias[EX];
+#pragma unroll
+  for (int e = 0; e < EX; ++e) {
+    const int i = tid + 256 * e, cc = c0 + i % CH;
+    bias[e] = (i < TB * CH && cc < C) ? ld_f((const T*)a.dt_bias + cc) : 0.f;
+  }
+  // the loads of a stage go to registers one stage ahead: they are in flight while the stage before is computed, so the only
+  // exposed memory latency is the first stage's.  Elements past the segment's end are zeros (dt = x = B = C = 0 leave the state).
+  float px[EX], pz[EX], pd[EX], pB[EB], pC[EB], pl[LMAX];
+  auto prefetch = [&](int t0) {
+    const int nb = min(TB, t_end - t0);
+#pragma unroll
+    for (int e = 0; e < EX; ++e) {
+      const int i = tid + 256 * e, t = i / CH, cc = c0 + i % CH;
+      const bool on = i < TB * CH && t < nb && cc < C;
+      px[e] = on ? ld_f((const T*)a.x + (long)(t0 + t) * a.ldx + cc) : 0.f;
+      pz[e] = on ? ld_f((const T*)a.z + (long)(t0 + t) * a.ldz + cc) : 0.f;
+      pd[e] = (on && !fused) ? a.dt_pre[(long)(t0 + t) * a.lddt + cc] : 0.f;
     }
-    for (int i = tid; i < TS * CH; i += 256) {
-      const int t = i / CH, cc = c0 + i % CH;
-      float dt = 0.f, xv = 0.f;
-      if (t < nb && cc < C) {
-        float pre;
-        if (a.dt_w) {
-          const float* lr = lows + t * R;
-          pre = 0.f;
-          if (wdt_lds) {
-            const float* wl = wdt + (i % CH) * (R + 1);
-#pragma unroll 8
-            for (int r = 0; r < R; ++r) pre = fmaf(wl[r], lr[r], pre);      // (unrolled: eight pairs of LDS reads in flight per wait)
-          } else {
-            const T* wr = (const T*)a.dt_w + (long)cc * R;
-#pragma unroll 8
-            for (int r = 0; r < R; ++r) pre = fmaf(ld_f(wr + r), lr[r], pre);
-          }
-        } else {
-          pre = a.dt_pre[(long)(t0 + t) * a.lddt + cc];
-        }
-        dt = softplus_f(pre + ld_f((const T*)a.dt_bias + cc));
-        xv = ld_f((const T*)a.x + (long)(t0 + t) * a.ldx + cc);
+#pragma unroll
+    for (int e = 0; e < EB; ++e) {
+      const int i = tid + 256 * e, t = i / NP, n = i % NP;
+      const bool on = i < TB * NP && t < nb && n < N;
+      pB[e] = on ? a.B[(long)(t0 + t) * a.ldbc + n] : 0.f;
+      pC[e] = on ? a.Cm[(long)(t0 + t) * a.ldbc + n] : 0.f;
+    }
+    if (fused) {
+#pragma unroll
+      for (int e = 0; e < LMAX; ++e) {
+        const int i = tid + 256 * e;
+        pl[e] = i < nb * R ? a.dt_low[(long)(t0 + i / R) * a.lddt + i % R] : 0.f;
       }
-      dts[i] = dt;
-      xs[i] = xv;
     }
-    for (int i = tid; i < TS * NP; i += 256) {
-      const int t = i / NP, n = i % NP;
-      const bool on = t < nb && n < N;
-      Bs[i] = on ? a.B[(long)(t0 + t) * a.ldbc + n] : 0.f;
-      Cs[i] = on ? a.Cm[(long)(t0 + t) * a.ldbc + n] : 0.f;
+  };
+  prefetch(t_begin);
+  for (int t0 = t_begin; t0 < t_end; t0 += TB) {
+    const int nb = min(TB, t_end - t0);
+#pragma unroll
+    for (int e = 0; e < EX; ++e) {
+      const int i = tid + 256 * e;
+      if (i < TB * CH) {
+        xs[i] = px[e];
+        zs[i] = pz[e];
+      }
+    }
+#pragma unroll
+    for (int e = 0; e < EB; ++e) {
+      const int i = tid + 256 * e;
+      if (i < TB * NP) {
+        Bs[i] = pB[e];
+        Cs[i] = pC[e];
+      }
+    }
+    if (fused) {
+#pragma unroll
+      for (int e = 0; e < LMAX; ++e) {
+        const int i = tid + 256 * e;
+        if (i < nb * R) lows[i] = pl[e];
+      }
+    }
+    float dpre[EX];
+#pragma unroll
+    for (int e = 0; e < EX; ++e) dpre[e] = pd[e];
+    __syncthreads();
+    if (t0 + TB < t_end) prefetch(t0 + TB);
+    // step sizes: softplus once per (token, channel); with W_dt given, its dot with the staged low-rank row first
+#pragma unroll
+    for (int e = 0; e < EX; ++e) {
+      const int i = tid + 256 * e, t = i / CH, cc = c0 + i % CH;
+      if (i < TB * CH) {
+        float dt = 0.f;
+        if (t < nb && cc < C) {
+          float pre = dpre[e];
+          if (fused) {
+            const float* lr = lows + t * R;
+            pre = 0.f;
+            if (wdt_lds) {
+              const float* wl = wdt + (i % CH) * (R + 1);
+#pragma unroll 8
+              for (int r = 0; r < R; ++r) pre = fmaf(wl[r], lr[r], pre);      // (unrolled: eight pairs of LDS reads in flight per wait)
+            } else {
+              const T* wr = (const T*)a.dt_w + (long)cc * R;
+#pragma unroll 8
+              for (int r = 0; r < R; ++r) pre = fmaf(ld_f(wr + r), lr[r], pre);
+            }
+          }
+          dt = softplus_f(pre + bias[e]);
+        }
+        dts[i] = dt;
+      }
     }
     __syncthreads();
     {
@@ -147,7 +203,7 @@ __global__ __launch_bounds__(256) void selective_scan_kernel(vlm_selective_scan_
     for (int i = tid; i < nb * CH; i += 256) {
       const int t = i / CH, cc = c0 + i % CH;
       if (cc < C) {
-        const float zv = ld_f((const T*)a.z + (long)(t0 + t) * a.ldz + cc);
+        const float zv = zs[i];
         st_f((T*)a.out + (long)(t0 + t) * a.ldo + cc, ys[i] * (zv / (1.f + expf(-zv))));
       }
     }
@@ -177,7 +233,7 @@ int run(const vlm_selective_scan_args& a, int nseg, int maxlen, hipStream_t st) 
   int P = 1;
   while (P * NS < a.N) P <<= 1;
   const int CH = 256 / P;
-  if ((size_t)TB * (3 * CH + 2 * P * NS + (a.dt_w ? a.R : 0)) * sizeof(float) > 64 * 1024 || (a.C + CH - 1) / CH > 65535) return VLM_ERR_SHAPE;
+  if ((size_t)TB * (3 * CH + 2 * P * NS + (a.dt_w ? a.R : 0)) * sizeof(float) > 64 * 1024 || (a.dt_w && a.R > 16 * LMAX) || (a.C + CH - 1) / CH > 65535) return VLM_ERR_SHAPE;
   if (NS == 2) launch<T, 64, 2>(a, nseg, maxlen, st);
   else if (NS == 4) launch<T, 64, 4>(a, nseg, maxlen, st);
   else if (P == 1) launch<T, 1, 1>(a, nseg, maxlen, st);
