@@ -106,7 +106,11 @@ __global__ __launch_bounds__(256) void selective_scan_kernel(vlm_selective_scan_
 #pragma unroll
       for (int e = 0; e < LMAX; ++e) {
         const int i = tid + 256 * e;
-        pl[e] = i < nb * R ? a.dt_low[(long)(t0 + i / R) * a.lddt + i % R] : 0.f;
+        pl[e] = 0.f;
+        if (i < nb * R) {                     // (a branch, not a select: the division stays out of the trips a short stage does not need)
+          const int t = i / R;
+          pl[e] = a.dt_low[(long)(t0 + t) * a.lddt + (i - t * R)];
+        }
       }
     }
   };
